@@ -273,6 +273,8 @@ struct HeadPrepArgs {
     float eps;
     int n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode;
     int page_tokens, max_blocks, write_kv, pairing;
+    const float* q_scale;    // [H] or null: a factor a query head on the rotated q (a temperature a head on its scores)
+    int ld;                  // row stride of qkv (at least its width: further columns of the projection may follow v)
 };
 
 template <typename T>
@@ -285,7 +287,7 @@ __global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs
     if (!is_q && !a.write_kv) return;
     const int g = hh - H;
     const int col0 = is_q ? hh * D : H * D + g * D;
-    const float* row = a.qkv + (size_t)t * width;
+    const float* row = a.qkv + (size_t)t * (a.ld > width ? a.ld : width);
     const int p = a.pos[t];
     float x[ATT_PREP_MAX_D / 64];
     float ss = 0.0f;
@@ -316,6 +318,7 @@ __global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs
         slot = p % a.page_tokens;
     }
     const size_t head_at = (size_t)page * G + g;
+    const float q_factor = is_q && a.q_scale ? a.q_scale[hh] : 1.0f;
 #pragma unroll
     for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
@@ -328,7 +331,7 @@ __global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs
             const float c = cs[pair], sn = cs[half + pair];
             y = first ? fmaf(-other, sn, y * c) : fmaf(other, sn, y * c);
         }
-        if (is_q) st((T*)a.q_out + (size_t)t * H * D + col0 + d, y);
+        if (is_q) st((T*)a.q_out + (size_t)t * H * D + col0 + d, a.q_scale ? y * q_factor : y);
         else st((T*)a.k_cache + (head_at * a.page_tokens + slot) * D + d, y);
     }
     if (!is_q) {
@@ -341,18 +344,42 @@ __global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs
 extern "C" int llmx_head_norm_rope_kvwrite(const float* qkv, const float* bias, const float* q_weight, const float* k_weight, const float* cos_sin,
                                            const int* pos, const int* row_entry, const int* tables, void* q_out, void* k_cache, void* v_cache,
                                            int dtype, float eps, int rows, int n_heads, int n_kv_heads, int head_dim, int v_dim, int rotary_dim,
-                                           int norm_mode, int page_tokens, int max_blocks, int write_kv, int pairing, hipStream_t stream) {
+                                           int norm_mode, int page_tokens, int max_blocks, int write_kv, int pairing, const float* q_scale,
+                                           int ld, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_HEAD) return -2;
     if (pairing != ROPE_HALVES && pairing != ROPE_INTERLEAVED) return -2;
     if (head_dim < 1 || head_dim > ATT_PREP_MAX_D || v_dim < 1 || rotary_dim > head_dim || rotary_dim % 2) return -2;
     if (norm_mode == QKNORM_HEAD && (!q_weight || !k_weight)) return -2;
     HeadPrepArgs a{qkv, bias, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
-                   n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, pairing};
+                   n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, pairing, q_scale, ld};
     llmx_note_launch(LK_HEAD_NORM_ROPE_KVWRITE);
     const dim3 grid(rows, n_heads + n_kv_heads);
     if (dtype == LLMX_F32) hipLaunchKernelGGL(head_norm_rope_kvwrite_kernel<float>, grid, dim3(64), 0, stream, a);
     else hipLaunchKernelGGL(head_norm_rope_kvwrite_kernel<bf16_t>, grid, dim3(64), 0, stream, a);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// A sigmoid gate a head on the attention's result, in place: o[t, h*V + d] *= sigmoid(gate[t*ldg + h]); the gate's logits
+// are float32 columns of a wider projection (row stride ldg).
+template <typename T>
+__global__ void __launch_bounds__(256) gate_heads_kernel(T* __restrict__ o, const float* __restrict__ gate, int ldg, int H, int V, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    const size_t t = at / ((size_t)H * V);
+    const int h = (int)((at / (size_t)V) % (size_t)H);
+    st(o + at, ld(o + at) * sigmoid_f(gate[t * ldg + h]));
+}
+
+extern "C" int llmx_gate_heads(void* o, int dtype, const float* gate, int ldg, int rows, int H, int V, hipStream_t stream) {
+    if (rows <= 0 || H <= 0 || V <= 0) return 0;
+    if (!gate || ldg < H) return -2;
+    llmx_note_launch(LK_GATE_HEADS);
+    const size_t total = (size_t)rows * H * V;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (dtype == LLMX_F32) hipLaunchKernelGGL(gate_heads_kernel<float>, grid, dim3(256), 0, stream, (float*)o, gate, ldg, H, V, total);
+    else hipLaunchKernelGGL(gate_heads_kernel<bf16_t>, grid, dim3(256), 0, stream, (bf16_t*)o, gate, ldg, H, V, total);
     return LLMX_CHECK_LAUNCH();
 }
 

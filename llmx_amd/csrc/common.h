@@ -268,4 +268,21 @@ struct ActFn {
     }
 };
 
+// A gated unit of two pre-activations (gate, up), as the products' gated epilogue and the kernel of its own compute it.
+// SILU: silu(gate) * up.  CLAMPED: g = min(gate, limit), u = clamp(up, -limit, limit); g sigmoid(1.702 g) (u + 1).
+enum : int { LLMX_GLU_SILU = 0, LLMX_GLU_CLAMPED = 1 };
+__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
+struct GluFn {
+    int kind;
+    float limit;
+    __device__ __forceinline__ GluFn(int kind_, float limit_) : kind(kind_), limit(limit_) {}
+    __device__ __forceinline__ float operator()(float gate, float up) const {
+        if (kind == LLMX_GLU_CLAMPED) {
+            const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+            return (g / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
+        }
+        return (gate / (1.0f + expf(-gate))) * up;
+    }
+};
+
 #define LLMX_CHECK_LAUNCH() (int)hipGetLastError()

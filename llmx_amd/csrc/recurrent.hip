@@ -21,7 +21,6 @@ struct ScanArgs {
     int W;
 };
 
-__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 #define SCAN_AHEAD 8
 template <typename TO>

@@ -142,3 +142,102 @@ extern "C" int llmx_act_gelu_gather(const float* z, const void* table, int table
 #undef LLMX_GG
     return LLMX_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------------------
+// x[t,:] = (x[t,:] + rows[t,:]) + vec[:]: what a repeated run of layers adds to the residual before a pass (rows: a kept
+// copy of earlier rows, or null; vec: the pass's own vector).
+__global__ void __launch_bounds__(256) add_rows_vector_kernel(float* __restrict__ x, const float* __restrict__ rows, const float* __restrict__ vec,
+                                                            int n, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    float v = x[at];
+    if (rows) v = v + rows[at];
+    if (vec) v = v + vec[(int)(at % (size_t)n)];
+    x[at] = v;
+}
+
+extern "C" int llmx_add_rows_vector(float* x, const float* rows, const float* vec, int n_rows, int n, hipStream_t stream) {
+    if (n_rows <= 0 || n <= 0) return 0;
+    llmx_note_launch(LK_ADD_ROWS_VECTOR);
+    const size_t total = (size_t)n_rows * n;
+    hipLaunchKernelGGL(add_rows_vector_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, rows, vec, n, total);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// A polynomial of unit-RMS powers between two products: with U(v) = v / sqrt(mean(v^2) + eps) over a row,
+// out = a U(z) + b U(z^2) + c U(z^3) + e, powers element by element, (a, b, c, e) four numbers on the device.  A block a
+// row: the sums of z^2, z^4 and z^6 in one pass (each in the fixed order of strided_squares and block_sum), then the
+// row again (it is still in the caches).  Everything float32; only the result is stored in the activation type.
+#define POLY_THREADS 256
+template <typename TO>
+__global__ void __launch_bounds__(POLY_THREADS) polynorm_kernel(const float* __restrict__ z, const float* __restrict__ abce, float eps,
+                                                              TO* __restrict__ out, int n) {
+    __shared__ float scratch[POLY_THREADS / 64];
+    const int r = blockIdx.x;
+    const float* row = z + (size_t)r * n;
+    const float a = abce[0], b = abce[1], c = abce[2], e = abce[3];
+    float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 4 * POLY_THREADS) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * POLY_THREADS < n ? row[i + u * POLY_THREADS] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float p2 = v[u] * v[u], p3 = p2 * v[u];
+            s2 = fmaf(v[u], v[u], s2);
+            s4 = fmaf(p2, p2, s4);
+            s6 = fmaf(p3, p3, s6);
+        }
+    }
+    s2 = block_sum<POLY_THREADS / 64>(s2, scratch);
+    s4 = block_sum<POLY_THREADS / 64>(s4, scratch);
+    s6 = block_sum<POLY_THREADS / 64>(s6, scratch);
+    const float r1 = a / sqrtf(s2 / (float)n + eps), r2 = b / sqrtf(s4 / (float)n + eps), r3 = c / sqrtf(s6 / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += POLY_THREADS) {
+        const float v = row[i], p2 = v * v;
+        st(out + (size_t)r * n + i, ((v * r1 + p2 * r2) + (p2 * v) * r3) + e);
+    }
+}
+
+extern "C" int llmx_act_polynorm(const float* z, const float* abce, float eps, void* out, int out_dtype, int rows, int n, hipStream_t stream) {
+    if (rows <= 0 || n <= 0) return 0;
+    llmx_note_launch(LK_ACT_POLYNORM);
+    if (out_dtype == LLMX_F32) hipLaunchKernelGGL(polynorm_kernel<float>, dim3(rows), dim3(POLY_THREADS), 0, stream, z, abce, eps, (float*)out, n);
+    else hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(rows), dim3(POLY_THREADS), 0, stream, z, abce, eps, (bf16_t*)out, n);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// A gated unit between two products, as a kernel of its own (GluFn: silu(gate) * up, or the clamped form): a row of `pre`
+// holds n gate values, then n up values (row stride ld); with s = row_scale[p] (a factor on the row's *input*, which the first
+// product being linear is a factor on both pre-activations; null: 1): out = unit(s gate, s up), times
+// sigmoid(row_gate[p * row_gate_ld]) where a gate logit a row is given.
+template <typename TO>
+__global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ pre, int ld, const float* __restrict__ row_scale,
+                                                        const float* __restrict__ row_gate, int row_gate_ld, int kind, float limit, TO* __restrict__ out,
+                                                        int n, size_t total) {
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    const size_t p = at / (size_t)n;
+    const int j = (int)(at % (size_t)n);
+    const GluFn glu(kind, limit);
+    const float s = row_scale ? row_scale[p] : 1.0f;
+    float y = glu(pre[p * ld + j] * s, pre[p * ld + n + j] * s);
+    if (row_gate) y = y * sigmoid_f(row_gate[p * row_gate_ld]);
+    st(out + at, y);
+}
+
+extern "C" int llmx_act_glu(const float* pre, int ld, const float* row_scale, const float* row_gate, int row_gate_ld, int kind, float limit,
+                            void* out, int out_dtype, int rows, int n, hipStream_t stream) {
+    if (rows <= 0 || n <= 0) return 0;
+    if (ld < 2 * n || (kind != LLMX_GLU_SILU && kind != LLMX_GLU_CLAMPED) || (kind == LLMX_GLU_CLAMPED && !(limit > 0.0f))) return -2;
+    llmx_note_launch(LK_ACT_GLU);
+    const size_t total = (size_t)rows * n;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (out_dtype == LLMX_F32)
+        hipLaunchKernelGGL(glu_kernel<float>, grid, dim3(256), 0, stream, pre, ld, row_scale, row_gate, row_gate_ld, kind, limit, (float*)out, n, total);
+    else
+        hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, dim3(256), 0, stream, pre, ld, row_scale, row_gate, row_gate_ld, kind, limit, (bf16_t*)out, n, total);
+    return LLMX_CHECK_LAUNCH();
+}

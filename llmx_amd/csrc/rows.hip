@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(float* __restrict__ x,
         for (int u = 0; u < 8; ++u) yv[u] = j0 + u < k ? y[((size_t)t * k + j0 + u) * width + i] : 0.0f;
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-            if (j0 + u < k && ids[t * k + j0 + u] >= 0) s += w[t * k + j0 + u] * yv[u];
+            if (j0 + u < k && ids[t * k + j0 + u] >= 0) s += (w ? w[t * k + j0 + u] : 1.0f) * yv[u];
     }
     *o = accumulate ? old + s : s;
 }
@@ -128,7 +128,7 @@ __global__ void __launch_bounds__(256) moe_combine4_kernel(float* __restrict__ x
         for (int u = 0; u < 8; ++u) {
             const int j = j0 + u;
             const bool in = j < k && ids[t * k + j] >= 0;
-            wj[u] = in ? w[t * k + j] : 0.0f;
+            wj[u] = in ? (w ? w[t * k + j] : 1.0f) : 0.0f;
             v[u] = in ? *reinterpret_cast<const f32x4_t*>(y + ((size_t)t * k + j) * width + i) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
         }
 #pragma unroll

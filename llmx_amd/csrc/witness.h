@@ -73,7 +73,11 @@
     X(DELTA_PREP, "delta_prep")                                                                                           \
     X(SIGMOID_ROOT, "sigmoid_root")                                                                                       \
     X(STATE_SCAN, "state_scan")                                                                                           \
-    X(HEAD_NORM_GATE, "head_norm_gate")
+    X(HEAD_NORM_GATE, "head_norm_gate")                                                                                   \
+    X(ADD_ROWS_VECTOR, "add_rows_vector")                                                                                 \
+    X(ACT_POLYNORM, "act.polynorm")                                                                                       \
+    X(ACT_GLU, "act.glu")                                                                                                 \
+    X(GATE_HEADS, "gate_heads")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

@@ -411,8 +411,14 @@ class Engine:
         T, E = step.rows, self.spec.hidden_size
         x = step.buf("residual", (T, E), torch.float32)
         self.model.embedding.forward(step, x)
+        kept = None
+        if any(p.wants_embedding for p in self.model.inputs):     # a residual input adds the embedding's rows again later
+            kept = step.buf("embedding.rows", (T, E), torch.float32)
+            self.model.embedding.forward(step, kept)
         for i, (entry, cache) in enumerate(zip(self.spec.run_order, self._layer_caches)):
             step.run_index = i
+            if entry.before is not None:
+                self.model.inputs[entry.before].forward(step, x, kept)
             self.model.blocks[entry.layer].forward(step, x, cache)
             if step.observer is not None:
                 step.observe("layer", run_index=i, residual=x)

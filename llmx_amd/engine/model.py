@@ -27,12 +27,13 @@ class BuiltModel:
         self.blocks = [build_block(b, ctx) for b in spec.blocks]
         self.final_norm = build_part("norm", spec.final_norm, ctx)
         self.head = build_part("head", spec.head, ctx)
+        self.inputs = [build_part("residual_input", p, ctx) for p in spec.inputs]
 
     def parts(self):
         out = [self.embedding]
         for b in self.blocks:
             out.extend(b.parts())
-        out += [self.final_norm, self.head]
+        out += [self.final_norm, self.head] + self.inputs
         # a part made of parts (mixers side by side) is followed by its members, which list and take their own tensors
         at = 0
         while at < len(out):

@@ -75,7 +75,11 @@ def _declare(h) -> None:
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P],
-        "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P],
+        "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P, I, P],
+        "llmx_gate_heads": [P, I, P, I, I, I, I, P],
+        "llmx_add_rows_vector": [P, P, P, I, I, P],
+        "llmx_act_polynorm": [P, P, F, P, I, I, I, P],
+        "llmx_act_glu": [P, I, P, P, I, I, F, P, I, I, I, P],
         "llmx_layernorm": [P, P, P, F, P, I, P, I, I, P],
         "llmx_layernorm_add": [P, P, P, F, P, I, I, I, P],
         "llmx_cast_rows": [P, P, I, L, P],
@@ -216,6 +220,52 @@ def rmsnorm_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: flo
     rows, n = x.shape
     _check(lib().llmx_rmsnorm_add(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, (rows, n)), _dev(weight, "weight", torch.float32, (n,)),
                                   float(eps), rows, n, _stream()), "rmsnorm_add")
+
+
+def add_rows_vector(x: torch.Tensor, rows: Optional[torch.Tensor], vec: Optional[torch.Tensor]) -> None:
+    """x[t] = (x[t] + rows[t]) + vec, float32; rows [T, n] and vec [n] may each be None."""
+    T, n = x.shape
+    _check(lib().llmx_add_rows_vector(_dev(x, "x", torch.float32), _dev(rows, "rows", torch.float32, (T, n)), _dev(vec, "vec", torch.float32, (n,)),
+                                      T, n, _stream()), "add_rows_vector")
+
+
+def act_polynorm(z: torch.Tensor, abce: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """out = a U(z) + b U(z^2) + c U(z^3) + e over float32 rows z [T, n], U(v) = v / sqrt(mean(v^2) + eps) a row, powers
+    element by element; abce = (a, b, c, e) float32 on the device."""
+    rows, n = z.shape
+    _check(lib().llmx_act_polynorm(_dev(z, "z", torch.float32), _dev(abce, "abce", torch.float32, (4,)), float(eps),
+                                   _dev(out, "out", shape=(rows, n)), _code(out.dtype), rows, n, _stream()), "act_polynorm")
+
+
+GLU_SILU, GLU_CLAMPED = 0, 1
+
+
+class Glu:
+    """The gated unit of a product's gated epilogue (EPI_SWIGLU) or of `act_glu`.  kind GLU_SILU: silu(gate) * up; GLU_CLAMPED:
+    g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1).  row_scale (float32 [rows of c]; None: 1):
+    a factor on both pre-activations of a row (a weight on what the product reads, the product being linear); row_gate (a
+    float32 view [rows of c, 1], rows possibly strided; None: none): the row's result is multiplied by sigmoid(row_gate)."""
+
+    def __init__(self, kind: int = GLU_SILU, limit: float = 0.0, row_scale: Optional[torch.Tensor] = None,
+                 row_gate: Optional[torch.Tensor] = None):
+        if kind not in (GLU_SILU, GLU_CLAMPED) or (kind == GLU_CLAMPED and not limit > 0.0):
+            raise KernelError("a gated unit is GLU_SILU or GLU_CLAMPED, the clamped one with a positive limit")
+        self.kind, self.limit, self.row_scale, self.row_gate = int(kind), float(limit), row_scale, row_gate
+
+    @property
+    def plain(self) -> bool:
+        return self.kind == GLU_SILU and self.row_scale is None and self.row_gate is None
+
+
+def act_glu(pre: torch.Tensor, glu: Glu, out: torch.Tensor) -> None:
+    """out[p] = unit(s gate, s up) (* sigmoid(row_gate[p])), where row p of the float32 `pre` [P, >= 2n] holds n gate values,
+    then n up values, and s = glu.row_scale[p]: the gated unit as a kernel of its own."""
+    P, n = out.shape
+    if pre.dim() != 2 or pre.shape[0] != P or pre.shape[1] < 2 * n:
+        raise KernelError(f"act_glu: pre-activations {tuple(pre.shape)} do not hold {P} rows of {n} gate and {n} up values")
+    gate_at, gate_ld = _rows_view(glu.row_gate, "row_gate", P, 1) if glu.row_gate is not None else (0, 0)
+    _check(lib().llmx_act_glu(_dev(pre, "pre", torch.float32), pre.shape[1], _dev(glu.row_scale, "row_scale", torch.float32, (P,)),
+                              gate_at, gate_ld, glu.kind, glu.limit, _dev(out, "out"), _code(out.dtype), P, n, _stream()), "act_glu")
 
 
 def act_xielu(z: torch.Tensor, pq: torch.Tensor, out: torch.Tensor) -> None:
@@ -696,14 +746,37 @@ def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
 ACT_NONE, ACT_XIELU = 0, 1      # activations a storing product can apply to what it stores
 
 
-def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False, scratch=None, act=None) -> None:
+def _scratch_now(device):
+    """Storage for a caller that brings no step workspace: allocated at the call."""
+    return lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=device)
+
+
+def _glu_apart(glu: Optional["Glu"], epilogue: int) -> bool:
+    """Whether a gated product runs as a storing product followed by the unit's own kernel."""
+    if glu is None:
+        return False
+    if epilogue != EPI_SWIGLU:
+        raise KernelError("a gated unit goes with the gated epilogue")
+    return not glu.plain
+
+
+def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False, scratch=None, act=None,
+         glu: Optional["Glu"] = None) -> None:
     """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T).
     `a` may be NormedRows where gemm_takes_normed_rows says so: the product reads bfloat16(norm(x)).
     `scratch(name, shape, dtype)` gives storage that lives as long as the caller's step (a step's workspace): with it,
     products of some tens of rows multiply K's runs in workgroups of their own; the bits are the same either way.
     `act` = (ACT_XIELU, params): with EPI_STORE, c = activation(a @ w^T), params the activation's numbers on the device
-    (xIELU: float32 (p, q)); the bits of the product followed by the activation's own kernel (act_xielu)."""
+    (xIELU: float32 (p, q)); the bits of the product followed by the activation's own kernel (act_xielu).
+    `glu`: the gated epilogue's unit (see Glu); None: silu(gate) * up."""
     M, K = a.shape
+    if _glu_apart(glu, epilogue):
+        if isinstance(a, NormedRows):
+            raise KernelError("gemm: normed rows are not taken with this gated unit")
+        pre = (scratch or _scratch_now(a.device))("gemm.glu_pre", (M, w.shape[0]), torch.float32)
+        gemm(a, w, pre, EPI_STORE, force_generic, scratch)
+        act_glu(pre, glu, c)
+        return
     act_args = (0, 0)
     if act is not None:
         if epilogue != EPI_STORE or act[0] != ACT_XIELU:
@@ -747,7 +820,8 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
 
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
                  epilogue: int = EPI_STORE, active: Optional[torch.Tensor] = None, n_active: Optional[torch.Tensor] = None,
-                 token_rows: Optional[int] = None, force_generic: bool = False, tile_stats: Optional[torch.Tensor] = None) -> None:
+                 token_rows: Optional[int] = None, force_generic: bool = False, tile_stats: Optional[torch.Tensor] = None,
+                 glu: Optional["Glu"] = None, scratch=None) -> None:
     """For each group g: rows p in pairs[offsets[g]:offsets[g+1]] get c[p] = a[p // a_div] @ w[g]^T.
 
     With EPI_SWIGLU w[g] holds gate rows then up rows and c[p] = silu(gate) * up.  `active` / `n_active` (from
@@ -755,6 +829,13 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
     count) take the weight-streaming kernel.
     """
     G, NW, K = w.shape
+    if _glu_apart(glu, epilogue):
+        if isinstance(a, NormedRows):
+            raise KernelError("grouped_gemm: normed rows are not taken with this gated unit")
+        pre = (scratch or _scratch_now(a.device))("grouped_gemm.glu_pre", (c.shape[0], NW), torch.float32)
+        grouped_gemm(a, w, pre, offsets, pairs, a_div, EPI_STORE, active, n_active, token_rows, force_generic, tile_stats)
+        act_glu(pre, glu, c)
+        return
     N = NW // 2 if epilogue == EPI_SWIGLU else NW
     if a.shape[1] != K or c.shape[1] != N:
         raise KernelError(f"grouped_gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
@@ -821,15 +902,20 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_w
 def head_norm_rope_kvwrite(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
                            cos_sin: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor, tables: torch.Tensor, q_out: torch.Tensor,
                            k_cache: torch.Tensor, v_cache: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, head_dim: int,
-                           rotary_dim: int, norm_mode: int, write_kv: bool = True, pairing: int = ROPE_HALVES) -> None:
+                           rotary_dim: int, norm_mode: int, write_kv: bool = True, pairing: int = ROPE_HALVES,
+                           q_scale: Optional[torch.Tensor] = None) -> None:
     """qknorm_rope_kvwrite for heads that are treated one by one: float32 rows qkv = q (H*D) | k (G*D) | v (G*VD) get the
-    projections' biases (`bias`, one vector of the row's width, or None), every q and k head an RMS norm over its own dims
+    projections' biases (`bias`, one vector of that width, or None), every q and k head an RMS norm over its own dims
     with a weight [D] shared by the heads (norm_mode QKNORM_HEAD; QKNORM_NONE: none), then the rotation; k and v go to the
-    row's page.  The value width VD is the value cache's and may differ from D."""
+    row's page.  The value width VD is the value cache's and may differ from D.  The rows may be wider than q | k | v (further
+    columns of one fused projection follow v and are left alone).  `q_scale` [H] float32: the rotated q of head h is
+    multiplied by q_scale[h] (a temperature a head on the scores, folded into the query)."""
     rows = qkv.shape[0]
     n_pages, hk, page_tokens, d = k_cache.shape
     v_dim = v_cache.shape[2]
     width = n_heads * head_dim + n_kv_heads * head_dim + n_kv_heads * v_dim
+    if qkv.dim() != 2 or qkv.shape[1] < width:
+        raise KernelError(f"head_norm_rope_kvwrite: rows of {tuple(qkv.shape)} do not hold q | k | v of {width} values")
     if ((hk, d) != (n_kv_heads, head_dim) or tuple(v_cache.shape) != (n_pages, hk, v_dim, page_tokens) or k_cache.dtype != q_out.dtype
             or v_cache.dtype != q_out.dtype):
         raise KernelError("head_norm_rope_kvwrite: cache shape or dtype does not fit the heads")
@@ -841,11 +927,22 @@ def head_norm_rope_kvwrite(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_we
         _dev(q_weight, "q_weight", torch.float32, (head_dim,))
         _dev(k_weight, "k_weight", torch.float32, (head_dim,))
     _check(lib().llmx_head_norm_rope_kvwrite(
-        _dev(qkv, "qkv", torch.float32, (rows, width)), _dev(bias, "bias", torch.float32, (width,)), _dev(q_weight, "q_weight"),
+        _dev(qkv, "qkv", torch.float32), _dev(bias, "bias", torch.float32, (width,)), _dev(q_weight, "q_weight"),
         _dev(k_weight, "k_weight"), _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (rows,)),
         _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32), _dev(q_out, "q_out", shape=(rows, n_heads * head_dim)),
         _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _code(q_out.dtype), float(eps), rows, n_heads, n_kv_heads, head_dim, v_dim,
-        rotary_dim, norm_mode, page_tokens, tables.shape[1], 1 if write_kv else 0, int(pairing), _stream()), "head_norm_rope_kvwrite")
+        rotary_dim, norm_mode, page_tokens, tables.shape[1], 1 if write_kv else 0, int(pairing),
+        _dev(q_scale, "q_scale", torch.float32, (n_heads,)), qkv.shape[1], _stream()), "head_norm_rope_kvwrite")
+
+
+def gate_heads(o: torch.Tensor, gate: torch.Tensor, heads: int) -> None:
+    """o[t, h*V + d] *= sigmoid(gate[t, h]), in place; o [T, heads * V] in its own type, gate a float32 view [T, heads] whose
+    rows may be columns of a wider projection."""
+    rows, width = o.shape
+    if width % heads:
+        raise KernelError(f"gate_heads: rows of {width} values are not {heads} heads")
+    at, ldg = _rows_view(gate, "gate", rows, heads)
+    _check(lib().llmx_gate_heads(_dev(o, "o"), _code(o.dtype), at, ldg, rows, heads, width // heads, _stream()), "gate_heads")
 
 
 class AttentionPlan:
@@ -1047,7 +1144,8 @@ def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.T
     moe_align(ids, n_experts, counts, offsets, pairs, active, n_active, scratch, tile_stats)
 
 
-def moe_combine(x: torch.Tensor, y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, accumulate: bool = True) -> None:
+def moe_combine(x: torch.Tensor, y: torch.Tensor, ids: torch.Tensor, weights: Optional[torch.Tensor], accumulate: bool = True) -> None:
+    """x[t] (+)= sum over the row's slots j of weights[t, j] * y[t*k + j] in slot order (weights None: every weight 1)."""
     rows, width = x.shape
     k = ids.shape[1]
     _check(lib().llmx_moe_combine(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, (rows * k, width)),

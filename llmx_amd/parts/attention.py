@@ -22,13 +22,17 @@ _NORM_MODES = {"none": ops.QKNORM_NONE, "projection": ops.QKNORM_PROJECTION, "he
 
 # the names of an attention's tensors below its prefix; `names` in the parameters replaces any of them
 _NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "q_norm": "q_norm.weight",
-          "k_norm": "k_norm.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias"}
+          "k_norm": "k_norm.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+          "head_temperature": "head_temperature", "head_gate": "gate_proj.weight"}
 
 
 class Attention(Mixer):
     """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "head" | "none"), eps, window (None | int), position (PartSpec),
     scale (None: head_dim^-1/2; else the factor the scores are multiplied by), v_dim (a value head's width, head_dim by
-    default), bias (True: q, k, v and the output projection have biases), names ({role: name below the prefix})."""
+    default), bias (True: q, k, v and the output projection have biases; "qkv": q, k and v only), head_temperature (True: a
+    learned factor a query head on its scores, tensor [heads]; it is folded into the rotated query), head_gate (True: the
+    result of head h is multiplied by sigmoid(W_g x)_h, W_g [heads, hidden] reading the mixer's input; its rows ride in the
+    fused projection behind v), names ({role: name below the prefix})."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx: BuildContext):
@@ -59,7 +63,12 @@ class Attention(Mixer):
         self.v_dim = int(p["v_dim"]) if p.get("v_dim") is not None else self.head_dim
         if not 0 < self.v_dim <= MAX_HEAD_DIM:
             raise ValueError(f"attention: v_dim {self.v_dim} is outside what the attention kernels take (1 to {MAX_HEAD_DIM})")
+        if p.get("bias", False) not in (False, True, "qkv"):
+            raise ValueError(f"attention: bias {p.get('bias')!r} is not one of [False, True, 'qkv']")
         self.bias = bool(p.get("bias", False))
+        self.out_bias = p.get("bias", False) is True
+        self.head_temperature = bool(p.get("head_temperature", False))
+        self.head_gate = bool(p.get("head_gate", False))
         self.names = dict(_NAMES)
         unknown = set(p.get("names") or {}) - set(_NAMES)
         if unknown:
@@ -70,10 +79,12 @@ class Attention(Mixer):
         self.v_width = self.kv_heads * self.v_dim
         self.o_width = self.heads * self.v_dim
         # the plain case (one width, no biases, no norm a head) keeps the kernel that norms whole projections
-        self.by_head = self.norm_mode == ops.QKNORM_HEAD or self.bias or self.v_dim != self.head_dim
+        self.by_head = (self.norm_mode == ops.QKNORM_HEAD or self.bias or self.v_dim != self.head_dim or self.head_temperature
+                        or self.head_gate)
+        self.gate_width = self.heads if self.head_gate else 0
         if self.by_head and self.norm_mode == ops.QKNORM_PROJECTION:
             raise ValueError("attention: a norm over the whole projection goes with values as wide as keys and no biases")
-        self.wqkv = self.wo = self.q_norm = self.k_norm = self.b_qkv = self.b_o = None
+        self.wqkv = self.wo = self.q_norm = self.k_norm = self.b_qkv = self.b_o = self.temperature = None
 
     def cache_need(self):
         if self.v_dim == self.head_dim:
@@ -87,7 +98,7 @@ class Attention(Mixer):
     def tensor_specs(self, available):
         # one product for the three projections: the file's q, k and v go straight into the rows q | k | v of one tensor
         q, kv, vw = self.q_width, self.kv_width, self.v_width
-        fused, shape = self.name("qkv_proj.weight"), (q + kv + vw, self.hidden)
+        fused, shape = self.name("qkv_proj.weight"), (q + kv + vw + self.gate_width, self.hidden)
         specs = [
             TensorSpec(self.tensor("q"), (q, self.hidden), into=(fused, shape, (slice(0, q),))),
             TensorSpec(self.tensor("k"), (kv, self.hidden), into=(fused, shape, (slice(q, q + kv),))),
@@ -102,8 +113,13 @@ class Attention(Mixer):
             fused_b, shape_b = self.name("qkv_proj.bias"), (q + kv + vw,)
             specs += [TensorSpec(self.tensor("q_bias"), (q,), "bias", into=(fused_b, shape_b, (slice(0, q),))),
                       TensorSpec(self.tensor("k_bias"), (kv,), "bias", into=(fused_b, shape_b, (slice(q, q + kv),))),
-                      TensorSpec(self.tensor("v_bias"), (vw,), "bias", into=(fused_b, shape_b, (slice(q + kv, q + kv + vw),))),
-                      TensorSpec(self.tensor("o_bias"), (self.hidden,), "bias")]
+                      TensorSpec(self.tensor("v_bias"), (vw,), "bias", into=(fused_b, shape_b, (slice(q + kv, q + kv + vw),)))]
+            if self.out_bias:
+                specs.append(TensorSpec(self.tensor("o_bias"), (self.hidden,), "bias"))
+        if self.head_gate:
+            specs.append(TensorSpec(self.tensor("head_gate"), (self.heads, self.hidden), into=(fused, shape, (slice(q + kv + vw, q + kv + vw + self.heads),))))
+        if self.head_temperature:
+            specs.append(TensorSpec(self.tensor("head_temperature"), (self.heads,), "bias", dtype="float32", init=("uniform", 0.5, 1.5)))
         return specs
 
     def load(self, tensors):
@@ -114,7 +130,10 @@ class Attention(Mixer):
             self.k_norm = tensors[self.tensor("k_norm")]
         if self.bias:
             self.b_qkv = tensors[self.name("qkv_proj.bias")]
-            self.b_o = tensors[self.tensor("o_bias")]
+            if self.out_bias:
+                self.b_o = tensors[self.tensor("o_bias")]
+        if self.head_temperature:
+            self.temperature = tensors[self.tensor("head_temperature")]
 
     def output_bias(self):
         """The output projection's bias, which a caller that joins this mixer's result with others may add itself
@@ -143,7 +162,8 @@ class Attention(Mixer):
     def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None, add_output_bias=True):
         T = step.rows
         act = step.act_dtype
-        qkv = step.buf("attention.qkv", (T, self.q_width + self.kv_width + self.v_width), torch.float32)
+        qkv_width = self.q_width + self.kv_width + self.v_width
+        qkv = step.buf("attention.qkv", (T, qkv_width + self.gate_width), torch.float32)
         ops.gemm(h, self.wqkv, qkv, scratch=step.buf)
         q = step.buf("attention.q", (T, self.q_width), act)
         cos_sin, rotary = self.position.rotation()
@@ -151,7 +171,7 @@ class Attention(Mixer):
         if self.by_head:
             ops.head_norm_rope_kvwrite(qkv, self.b_qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k,
                                        cache.v, self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode,
-                                       write_kv=cache.writes, pairing=self.pairing)
+                                       write_kv=cache.writes, pairing=self.pairing, q_scale=self.temperature)
         else:
             ops.qknorm_rope_kvwrite(qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k, cache.v,
                                     self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes,
@@ -160,6 +180,8 @@ class Attention(Mixer):
         plan = self._plan(step) if self._mfma(act, cache.k.shape[2]) else None
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
                             window=int(self.window or 0), plan=plan, scratch=step.buf)
+        if self.head_gate:
+            ops.gate_heads(o, qkv[:, qkv_width:], self.heads)
         if self.b_o is not None and add_output_bias:
             y = step.buf("attention.projected", (T, self.hidden), torch.float32)
             ops.gemm(o, self.wo, y, scratch=step.buf)

@@ -162,6 +162,16 @@ class Embedding(Part):
         raise NotImplementedError
 
 
+class ResidualInput(Part):
+    """Something added to the residual between two run-order entries (before the entry that names it)."""
+    #: True when forward wants the embedding's rows as the step's first layer saw them; the engine then keeps a copy
+    wants_embedding = False
+
+    def forward(self, step, x: torch.Tensor, embedding_rows: Optional[torch.Tensor]) -> None:
+        """x (float32 [T, hidden]) += the part's addition; embedding_rows: float32 [T, hidden] when wanted, else None."""
+        raise NotImplementedError
+
+
 class Head(Part):
     def forward(self, step, rows: torch.Tensor, logits: torch.Tensor) -> None:
         """logits (float32 [W, vocab]) for the normed rows (activation type [W, hidden])."""
@@ -171,7 +181,7 @@ class Head(Part):
 # ---------------------------------------------------------------------------
 # registries: part name -> class
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {k: {} for k in ("norm", "position", "mixer", "feed_forward", "embedding", "head", "block",
-                                                                 "scale", "token_input")}
+                                                                 "scale", "token_input", "residual_input")}
 
 
 def register(family: str, kind: str, cls: Callable, replace: bool = False) -> None:

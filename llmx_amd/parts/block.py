@@ -6,6 +6,7 @@
 coordinate, and an optional per-layer token input after the sum.
 "outnorm": x += norm1(mixer(x)); x += norm2(ffn(x)): the sublayers read the residual itself and only their results are
 normed.
+"sandwich": x += norm1b(mixer(norm1(x))); x += norm2b(ffn(norm2(x))): a norm on both sides of each sublayer.
 """
 
 from __future__ import annotations
@@ -176,7 +177,48 @@ class OutNormBlock:
             step.shared("outnorm.copy", dict)["for"] = step.run_index + 1
 
 
+class SandwichBlock:
+    """x += mixer_post(mixer(mixer_norm(x))); x += ffn_post(ffn(ffn_norm(x))): a norm before and a norm after each
+    sublayer, the feed-forward (with both its norms) optional.  The slots: mixer_norm, mixer, ffn_norm, ffn; in `extra`:
+    "mixer_post" and "ffn_post" (family "norm", parts that have `add_into`: x += norm(y))."""
+    graph_safe = True
+
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        if (spec.ffn is None) != (spec.ffn_norm is None) or (spec.ffn is None) != ("ffn_post" not in spec.extra):
+            raise ValueError("sandwich block: a feed-forward comes with both its norms, and the norms with their feed-forward")
+        unknown = set(spec.extra) - {"mixer_post", "ffn_post"}
+        if unknown or "mixer_post" not in spec.extra:
+            raise ValueError(f"sandwich block: the extra slots are mixer_post and ffn_post, not {sorted(spec.extra)}")
+        for slot, (family, _) in spec.extra.items():
+            if family != "norm":
+                raise ValueError(f"sandwich block: {slot} is a part of family 'norm', not {family!r}")
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx)
+        self.mixer = build_part("mixer", spec.mixer, ctx)
+        self.mixer_post = build_part("norm", spec.extra["mixer_post"][1], ctx)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, ctx) if spec.ffn_norm is not None else None
+        self.ffn = build_part("feed_forward", spec.ffn, ctx) if spec.ffn is not None else None
+        self.ffn_post = build_part("norm", spec.extra["ffn_post"][1], ctx) if spec.ffn is not None else None
+        for n in (self.mixer_post, self.ffn_post):
+            if n is not None and not hasattr(n, "add_into"):
+                raise ValueError(f"sandwich block: the norm {n.kind!r} cannot join a result into the residual (no add_into)")
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post) if p is not None]
+
+    def forward(self, step, x: torch.Tensor, cache: LayerCache) -> None:
+        T, E = x.shape
+        y = step.buf("block.y", (T, E), torch.float32)
+        h, h32 = PreNormBlock.normed(step, self.mixer_norm, self.mixer, x)
+        self.mixer.forward(step, h, y, False, cache, h32)
+        self.mixer_post.add_into(step, x, y)
+        if self.ffn is not None:
+            h, h32 = PreNormBlock.normed(step, self.ffn_norm, self.ffn, x)
+            self.ffn.forward(step, h, y, False, h32)
+            self.ffn_post.add_into(step, x, y)
+
+
 register("block", "prenorm", PreNormBlock)
+register("block", "sandwich", SandwichBlock)
 register("block", "outnorm", OutNormBlock)
 register("block", "parallel", ParallelBlock)
 register("scale", "layer_scale", LayerScale)

@@ -28,6 +28,10 @@ _EXPERT_NAMES = {"router": "gate.weight", "correction_bias": "gate.e_score_corre
                  "expert_gate": "experts.{e}.gate_proj.weight", "expert_up": "experts.{e}.up_proj.weight",
                  "expert_down": "experts.{e}.down_proj.weight"}
 _GLU_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+# a shared expert's tensors below the routed feed-forward's prefix
+_EXPERT_NAMES.update({"shared_gate": "shared_expert.gate_proj.weight", "shared_up": "shared_expert.up_proj.weight",
+                      "shared_down": "shared_expert.down_proj.weight", "shared_switch": "shared_expert_gate.weight"})
+_UNITS = {"swiglu": ops.GLU_SILU, "clamped_glu": ops.GLU_CLAMPED}
 
 
 def _names(defaults: dict, given, what: str) -> dict:
@@ -42,7 +46,13 @@ def _names(defaults: dict, given, what: str) -> dict:
 class RoutedExperts(FeedForward):
     """params: hidden, experts, top_k, intermediate, score ("sigmoid" | "softmax"), correction_bias (bool: a bias on the pick
     keys only), logit_bias (bool: a bias that is part of the router's logits), normalize (bool), scale, names ({role: name
-    below the prefix}), files ("fused" | "per_expert": how a model folder of the design holds the experts, for when no file says).  score "softmax" with normalize "always" is the softmax over the picked logits alone, for any top_k."""
+    below the prefix}), files ("fused" | "per_expert": how a model folder of the design holds the experts, for when no file says).  score "softmax" with normalize "always" is the softmax over the picked logits alone, for any top_k.
+    unit ("swiglu", the default: silu(gate) * up | "clamped_glu": g = min(gate, limit), u = clamp(up, -limit, limit),
+    g sigmoid(1.702 g) (u + 1)) with limit; weight_on ("output", the default: the row's result is sum_j w_j expert_j(h) |
+    "input": sum_j expert_j(w_j h), the weight multiplying what the expert reads; the first product being linear, it is
+    applied to both pre-activations before the unit); shared ({intermediate, limit (for clamped_glu), switch (bool)}: an
+    expert of the same unit that every row runs, added to the routed sum, times sigmoid(W_switch h) (one number a row)
+    where it has a switch)."""
     graph_safe = True
 
     wants_f32_input = True
@@ -71,8 +81,24 @@ class RoutedExperts(FeedForward):
         if self.experts > MAX_EXPERTS or self.top_k > MAX_TOP_K:
             raise ValueError(f"routed experts: {self.experts} experts with {self.top_k} picks a token; the routing kernels take at most "
                              f"{MAX_EXPERTS} experts and {MAX_TOP_K} picks")
+        if p.get("unit", "swiglu") not in _UNITS:
+            raise ValueError(f"routed experts: unit {p.get('unit')!r} is not one of {sorted(_UNITS)}")
+        self.unit = _UNITS[p.get("unit", "swiglu")]
+        self.limit = float(p.get("limit") or 0.0)
+        if self.unit == ops.GLU_CLAMPED and not self.limit > 0.0:
+            raise ValueError("routed experts: the clamped unit needs a positive limit")
+        self.weight_on = str(p.get("weight_on", "output"))
+        if self.weight_on not in ("output", "input"):
+            raise ValueError(f"routed experts: weight_on {self.weight_on!r} is not one of ['input', 'output']")
+        shared = p.get("shared")
+        self.shared_width = int(shared["intermediate"]) if shared else 0
+        self.shared_limit = float(shared.get("limit") or 0.0) if shared else 0.0
+        self.shared_switch = bool(shared.get("switch", False)) if shared else False
+        if shared and (self.shared_width < 1 or (self.unit == ops.GLU_CLAMPED and not self.shared_limit > 0.0)):
+            raise ValueError("routed experts: a shared expert has an inner width of at least 1 and, for the clamped unit, a positive limit")
         self.per_expert = False
         self.w_router = self.bias = self.logit_bias = self.w_gate_up = self.w_down = None
+        self.w_shared_gate_up = self.w_shared_down = self.w_switch = None
 
     def tensor_specs(self, available):
         X, F, E = self.experts, self.intermediate, self.hidden
@@ -99,6 +125,14 @@ class RoutedExperts(FeedForward):
                           TensorSpec(nm("expert_down", e=e), (E, F), into=(down, (X, E, F), (e,)))]
         else:
             specs += [TensorSpec(fused, (X, 2 * F, E)), TensorSpec(nm("fused_down"), (X, E, F))]
+        if self.shared_width:
+            S = self.shared_width
+            shared = self.name("shared_gate_up")     # gate rows, then up rows, filled from the file's two tensors
+            specs += [TensorSpec(nm("shared_gate"), (S, E), into=(shared, (2 * S, E), (slice(0, S),))),
+                      TensorSpec(nm("shared_up"), (S, E), into=(shared, (2 * S, E), (slice(S, 2 * S),))),
+                      TensorSpec(nm("shared_down"), (E, S))]
+            if self.shared_switch:
+                specs.append(TensorSpec(nm("shared_switch"), (1, E), "router"))
         return specs
 
     def load(self, tensors):
@@ -110,8 +144,15 @@ class RoutedExperts(FeedForward):
         # per-expert files arrive fused too (see tensor_specs)
         self.w_gate_up = tensors[self.name(self.names["fused_gate_up"])]
         self.w_down = tensors[self.name(self.names["fused_down"])]
+        if self.shared_width:
+            self.w_shared_gate_up = tensors[self.name("shared_gate_up")]
+            self.w_shared_down = tensors[self.name(self.names["shared_down"])]
+            if self.shared_switch:
+                self.w_switch = tensors[self.name(self.names["shared_switch"])]
 
     def takes_deferred_norm(self, step):
+        if self.shared_width:      # the shared expert's products read the rows as tensors
+            return False
         return (ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU, grouped=True)
                 and ops.gemm_f32_takes_normed_rows(step.rows, self.w_router))
 
@@ -136,10 +177,23 @@ class RoutedExperts(FeedForward):
                              parts=parts, scratch=scratch, tile_stats=tile_stats, logit_bias=self.logit_bias)
         step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
-        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=tile_stats)
+        on_input = self.weight_on == "input"
+        glu = ops.Glu(self.unit, self.limit, weights.view(T * k) if on_input else None)
+        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=tile_stats,
+                         glu=glu, scratch=step.buf)
         y = step.buf("experts.y", (T * k, self.hidden), torch.float32)
         ops.grouped_gemm(act, self.w_down, y, offsets, pairs, 1, ops.EPI_STORE, active, n_active, token_rows=T, tile_stats=tile_stats)
-        ops.moe_combine(out, y, ids, weights, accumulate)
+        ops.moe_combine(out, y, ids, None if on_input else weights, accumulate)
+        if self.shared_width:
+            # the shared expert: its switch is a factor on the rows its second product reads (that product is linear), so the
+            # product can add straight into the routed sum
+            switch = None
+            if self.w_switch is not None:
+                switch = step.buf("experts.switch", (T, 1), torch.float32)
+                ops.gemm_f32(h32, self.w_switch, switch)
+            shared = step.buf("experts.shared_act", (T, self.shared_width), step.act_dtype)
+            ops.gemm(h, self.w_shared_gate_up, shared, ops.EPI_SWIGLU, glu=ops.Glu(self.unit, self.shared_limit, None, switch), scratch=step.buf)
+            ops.gemm(shared, self.w_shared_down, out, ops.EPI_ADD, scratch=step.buf)
 
 
 class DenseGLU(FeedForward):
@@ -175,8 +229,11 @@ class DenseGLU(FeedForward):
 
 
 class DenseAct(FeedForward):
-    """params: hidden, intermediate, activation ("xielu").  y = W_down act(W_up h); tensors <prefix>up, down, and for xIELU
-    <prefix>act = (p, q): act(z) = softplus(p) z^2 + z/2 for z > 0, (1/2 + softplus(q)) (e^z - 1 - z) + z/2 otherwise."""
+    """params: hidden, intermediate, activation ("xielu" | "polynorm"), eps (polynorm).  y = W_down act(W_up h); tensors
+    <prefix>up, down, and <prefix>act: for xIELU (p, q): act(z) = softplus(p) z^2 + z/2 for z > 0, (1/2 + softplus(q))
+    (e^z - 1 - z) + z/2 otherwise; for polynorm (a, b, c, e): act(z) = a U(z) + b U(z^2) + c U(z^3) + e with powers element by
+    element and U dividing a row of inner values by its root mean square (eps inside the root): it needs the whole row, so
+    it is a kernel of its own between the two products, in float32."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
@@ -184,14 +241,16 @@ class DenseAct(FeedForward):
         self.hidden = int(params["hidden"])
         self.intermediate = int(params["intermediate"])
         self.activation = str(params.get("activation", "xielu"))
-        if self.activation != "xielu":
-            raise ValueError(f"dense feed-forward: activation {self.activation!r} is not one of ['xielu']")
+        if self.activation not in ("xielu", "polynorm"):
+            raise ValueError(f"dense feed-forward: activation {self.activation!r} is not one of ['polynorm', 'xielu']")
+        self.eps = float(params.get("eps", 0.0))
         self.w_up = self.w_down = self.act = None
 
     def tensor_specs(self, available):
         F, E = self.intermediate, self.hidden
+        numbers = 2 if self.activation == "xielu" else 4
         return [TensorSpec(self.name("up"), (F, E)), TensorSpec(self.name("down"), (E, F)),
-                TensorSpec(self.name("act"), (2,), "bias", dtype="float32", init=("uniform", -1.0, 1.0))]
+                TensorSpec(self.name("act"), (numbers,), "bias", dtype="float32", init=("uniform", -1.0, 1.0))]
 
     def load(self, tensors):
         self.w_up = tensors[self.name("up")]
@@ -200,7 +259,12 @@ class DenseAct(FeedForward):
 
     def forward(self, step, h, out, accumulate, h32=None):
         a = step.buf("dense.act", (step.rows, self.intermediate), step.act_dtype)
-        ops.gemm(h, self.w_up, a, scratch=step.buf, act=(ops.ACT_XIELU, self.act))      # the activation in the product's epilogue
+        if self.activation == "polynorm":
+            z = step.buf("dense.pre", (step.rows, self.intermediate), torch.float32)
+            ops.gemm(h, self.w_up, z, scratch=step.buf)
+            ops.act_polynorm(z, self.act, self.eps, a)
+        else:
+            ops.gemm(h, self.w_up, a, scratch=step.buf, act=(ops.ACT_XIELU, self.act))      # the activation in the product's epilogue
         ops.gemm(a, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 

@@ -19,8 +19,10 @@ from .spec import TensorSpec
 class RMSNorm(Norm):
     """params: width, eps; gain ("vector", the default: one weight a coordinate; "scalar": the file holds one number for
     all coordinates); tensor (the name's last part, "weight" by default; "" when the prefix is the whole name); optional
-    (True: a norm that nothing runs, listed only so that a file which holds its tensor all the same is not refused).
-    Tensor: <prefix><tensor>, (width,) or ()."""
+    (True: a norm that nothing runs, listed only so that a file which holds its tensor all the same is not refused);
+    offset (0 by default; 1 for a weight that is stored around zero: the gain is offset + the stored weight, formed once
+    at load in float32).  Tensor: <prefix><tensor>, (width,) or ().  `add_into` is the form an arrangement uses that norms
+    a sublayer's result on its way into the residual."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
@@ -32,17 +34,22 @@ class RMSNorm(Norm):
             raise ValueError(f"norm gain {self.gain!r} is not one of ['scalar', 'vector']")
         self.tensor = str(params.get("tensor", "weight"))
         self.optional = bool(params.get("optional", False))
+        self.offset = float(params.get("offset", 0.0))
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self, available):
         if self.optional and self.name(self.tensor) not in available:
             return []
-        return [TensorSpec(self.name(self.tensor), (self.width,) if self.gain == "vector" else (), "norm")]
+        # random weights: the gain lies around 1 either way, so a stored weight with an offset lies around 1 - offset
+        init = ("normal", 1.0 - self.offset, 0.05) if self.offset else None
+        return [TensorSpec(self.name(self.tensor), (self.width,) if self.gain == "vector" else (), "norm", init=init)]
 
     def load(self, tensors):
         if self.optional and self.name(self.tensor) not in tensors:
             return
         w = tensors[self.name(self.tensor)]
+        if self.offset:
+            w = w + self.offset
         # one number for all coordinates is kept as a row of that number, which every norm kernel takes as it is
         self.weight = w if self.gain == "vector" else w.reshape(1).expand(self.width).contiguous()
 
@@ -51,6 +58,12 @@ class RMSNorm(Norm):
 
     def deferred(self, x):
         return ops.NormedRows(x, self.weight, self.eps)
+
+    def add_into(self, step, x, y, copy=None):
+        """x += norm(y); `copy` (optional) receives the new rows in its own type."""
+        ops.rmsnorm_add(x, y, self.weight, self.eps)
+        if copy is not None:
+            ops.cast_rows(x, copy)
 
 
 class LayerNorm(Norm):

@@ -81,21 +81,45 @@ def blended_frequencies(dims: int, base: float, scaling) -> tuple:
     return f / factor * ramp + f * (1.0 - ramp), 0.1 * float(np.log(factor)) + 1.0
 
 
+def wavelength_scaled_frequencies(dims: int, base: float, scaling) -> np.ndarray:
+    """Frequencies [dims/2] float64 rescaled by wavelength: f_i = base^(-2i/dims); with `scaling` = {factor, low, high,
+    original} and a pair's wavelength l = 2 pi / f: l < original/high keeps f; l > original/low gives f / factor; between
+    the two, s = (original/l - low) / (high - low) blends them, (1 - s) f / factor + s f.  No factor on cos and sin."""
+    i = np.arange(dims // 2, dtype=np.float64)
+    f = np.power(float(base), -2.0 * i / float(dims)) if dims else i
+    if not scaling:
+        return f
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+    low, high = float(scaling["low"]), float(scaling["high"])
+    if not (factor > 0.0 and original > 0.0 and low > 0.0 and high > low):
+        raise ValueError("rotary scaling: factor, original and low must be positive and high above low")
+    wavelength = 2.0 * np.pi / f
+    s = (original / wavelength - low) / (high - low)
+    blended = (1.0 - s) * f / factor + s * f
+    return np.where(wavelength < original / high, f, np.where(wavelength > original / low, f / factor, blended))
+
+
 def scaled_table(positions: int, dims: int, base: float, scaling) -> np.ndarray:
     """[positions, dims] float32: magnitude * cos of the dims/2 pairs' angles, then magnitude * sin.  The angle is the
     float32 product of the position and the float32 frequency; cos and sin are evaluated in float64 on it and rounded
     once, as `neox_table` does."""
     if dims == 0:
         return np.zeros((positions, 0), dtype=np.float32)
-    f, magnitude = blended_frequencies(dims, base, scaling)
+    if scaling and "low" in scaling:           # {factor, low, high, original}: rescaled by wavelength
+        # this form has no float32 recipe to follow: the angle is formed in float64 and only cos and sin are rounded
+        f = wavelength_scaled_frequencies(dims, base, scaling)
+        angle = np.arange(positions, dtype=np.float64)[:, None] * f[None, :]
+        return np.concatenate([np.cos(angle), np.sin(angle)], axis=1).astype(np.float32)
+    f, magnitude = blended_frequencies(dims, base, scaling)      # None, or {factor, original, fast, slow}
     pos = np.arange(positions, dtype=np.float32)[:, None]
     angle = (pos * f.astype(np.float32)[None, :]).astype(np.float32).astype(np.float64)
     return (np.concatenate([np.cos(angle), np.sin(angle)], axis=1) * magnitude).astype(np.float32)
 
 
 class ScaledRotary(PositionEncoding):
-    """Rotary pairs with an optional YaRN blend of the frequencies.  params: dims (even; the rotated dims), base, scaling
-    (None, or {factor, original, fast, slow}), pairing ("interleaved", the default here: dims 2i and 2i + 1; "halves")."""
+    """Rotary pairs with optionally rescaled frequencies.  params: dims (even; the rotated dims), base, scaling (None;
+    {factor, original, fast, slow}: the YaRN blend over the pair index with its factor on cos and sin; {factor, low, high,
+    original}: frequencies rescaled by wavelength, see `wavelength_scaled_frequencies`), pairing ("interleaved", the default here: dims 2i and 2i + 1; "halves")."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):

@@ -79,11 +79,14 @@ class RunEntry:
     """One item of the run order: run block `layer` with cache `cache`.
 
     A layer may be named by several entries (its weights run twice); two entries may name one cache, the later ones
-    with writes=False reading what the first wrote.
+    with writes=False reading what the first wrote.  `before`: the number of one of the model's residual inputs
+    (`ModelSpec.inputs`) that is added to the residual right before this entry's block runs (what a repeated run of
+    layers adds at the start of a pass); None: nothing.
     """
     layer: int
     cache: int
     writes: bool = True
+    before: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -164,11 +167,15 @@ class ModelSpec:
     head: PartSpec
     eos_token_id: Optional[int] = None
     bos_token_id: Optional[int] = None
+    #: parts of the family "residual_input" that run-order entries name by number (`RunEntry.before`)
+    inputs: List[PartSpec] = field(default_factory=list)
 
     def check(self) -> None:
         n_caches = 0
         writers = set()
         for e in self.run_order:
+            if e.before is not None and not 0 <= e.before < len(self.inputs):
+                raise ValueError(f"run order names residual input {e.before}, outside the model's {len(self.inputs)}")
             if not 0 <= e.layer < len(self.blocks):
                 raise ValueError(f"run order names layer {e.layer}, outside the model's {len(self.blocks)} layers")
             if e.writes:
