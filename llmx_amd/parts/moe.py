@@ -151,8 +151,8 @@ class RoutedExperts(FeedForward):
                 self.w_switch = tensors[self.name(self.names["shared_switch"])]
 
     def takes_deferred_norm(self, step):
-        if self.shared_width:      # the shared expert's products read the rows as tensors
-            return False
+        if self.shared_width or self.unit != ops.GLU_SILU or self.weight_on == "input":
+            return False           # the shared expert's products and the other gated units read the rows as tensors
         return (ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU, grouped=True)
                 and ops.gemm_f32_takes_normed_rows(step.rows, self.w_router))
 
