@@ -285,4 +285,30 @@ struct GluFn {
     }
 };
 
+// What a product's gated epilogue needs beyond its two accumulators: the unit, and two optional per-row values indexed by
+// the row of C: a factor on both pre-activations (a weight on the row's input: the product is linear) and a logit whose
+// sigmoid multiplies the row's result.  All zero: silu(gate) * up.
+struct GluArgs {
+    int kind;
+    float limit;
+    const float* row_scale;   // [rows of C] or null
+    const float* row_gate;    // [rows of C] with stride row_gate_ld, or null
+    int row_gate_ld;
+};
+struct GluRow {
+    GluFn fn;
+    float s, post;
+    bool scaled, gated;
+    __device__ __forceinline__ GluRow(const GluArgs& a, int row) : fn(a.kind, a.limit), s(1.0f), post(1.0f), scaled(a.row_scale != nullptr),
+                                                                  gated(a.row_gate != nullptr) {
+        if (scaled) s = a.row_scale[row];
+        if (gated) post = sigmoid_f(a.row_gate[(size_t)row * a.row_gate_ld]);
+    }
+    __device__ __forceinline__ float operator()(float gate, float up) const {
+        float y = scaled ? fn(gate * s, up * s) : fn(gate, up);
+        if (gated) y = y * post;
+        return y;
+    }
+};
+
 #define LLMX_CHECK_LAUNCH() (int)hipGetLastError()

@@ -28,6 +28,7 @@ struct GemmArgs {
     int up_offset;  // EPI_SWIGLU: W row n is the gate row, W row n + up_offset the up row
     int act;        // EPI_STORE: an activation applied to what is stored (LLMX_ACT_*), with its parameters on the device
     const float* act_params;
+    GluArgs glu;    // EPI_SWIGLU: the gated unit and its per-row values
 };
 
 template <typename TA, typename TW, typename TC, int EPI>
@@ -122,6 +123,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
         for (int i = 0; i < 4; ++i) {
             const int rc = rowsC[ty * 4 + i];
             if (rc < 0) continue;
+            const GluRow glu(g.glu, EPI == EPI_SWIGLU ? rc : 0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int n = n0 + tx * 4 + j;
@@ -129,8 +131,8 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs g) {
                 TC* c = C + (size_t)rc * g.ldc + n;
                 float v = acc[i][j];
                 if (EPI == EPI_SWIGLU) {
-                    // silu(g) * u with silu(x) = x / (1 + exp(-x))
-                    v = (v / (1.0f + expf(-v))) * accu[i][j];
+                    // the gated unit; by default silu(g) * u with silu(x) = x / (1 + exp(-x))
+                    v = glu(v, accu[i][j]);
                 } else if (EPI == EPI_ADD) {
                     v = ld(c) + v;
                 } else {
@@ -163,12 +165,15 @@ static int launch_c(const GemmArgs& g, int c_dtype, int epi, dim3 grid, hipStrea
 // dtype codes: 0 f32, 1 bf16.  n_groups == 0: dense product over M rows.  n_groups > 0: grouped (see GemmArgs).
 extern "C" int llmx_gemm_generic(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda,
                                  int ldw, int ldc, int epi, int n_groups, const int* group_offsets, const int* list, int a_div,
-                                 long w_group_stride, int up_offset, int act, const float* act_params, hipStream_t stream) {
+                                 long w_group_stride, int up_offset, int act, const float* act_params, int glu_kind, float glu_limit,
+                                 const float* glu_row_scale, const float* glu_row_gate, int glu_row_gate_ld, hipStream_t stream) {
     if (N <= 0 || K <= 0) return 0;
     if (n_groups == 0 && M <= 0) return 0;
     llmx_note_launch(n_groups ? LK_GEMM_GENERIC_GROUPED : LK_GEMM_GENERIC);
     GemmArgs g{A, W, C, M, N, K, lda, ldw, ldc, n_groups ? group_offsets : nullptr, list, a_div > 0 ? a_div : 1, w_group_stride, up_offset,
-               epi == EPI_STORE ? act : LLMX_ACT_NONE, act_params};
+               epi == EPI_STORE ? act : LLMX_ACT_NONE, act_params,
+               GluArgs{epi == EPI_SWIGLU ? glu_kind : LLMX_GLU_SILU, glu_limit, epi == EPI_SWIGLU ? glu_row_scale : nullptr,
+                       epi == EPI_SWIGLU ? glu_row_gate : nullptr, glu_row_gate_ld}};
     if (act != LLMX_ACT_NONE && (epi != EPI_STORE || !act_params)) return -2;
     dim3 grid;
     grid.x = (N + GT_BN - 1) / GT_BN;

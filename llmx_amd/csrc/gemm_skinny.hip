@@ -44,6 +44,7 @@ struct SkinnyArgs {
     // SK_STORE: an activation applied to what is stored (LLMX_ACT_*), with its parameters on the device
     int act;
     const float* act_params;
+    GluArgs glu;    // SK_SWIGLU: the gated unit and its per-row values
 };
 
 __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool in) {
@@ -224,11 +225,12 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
                 const int rc = rows_c[t * 16 + r];
                 if (rc < 0) continue;
                 TC* c = (TC*)g.C + (size_t)rc * g.ldc + n0 + 4 * kg;
+                const GluRow glu(g.glu, EPI == SK_SWIGLU ? rc : 0);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (n0 + 4 * kg + i >= g.N) continue;
                     float x = v[0][i];
-                    if (EPI == SK_SWIGLU) x = (x / (1.0f + expf(-x))) * v[1][i];
+                    if (EPI == SK_SWIGLU) x = glu(x, v[1][i]);
                     if (EPI == SK_ADD) x = c_old[t][i] + x;
                     if (EPI == SK_STORE && g.act != LLMX_ACT_NONE) x = ActFn(g.act, act_params)(x);
                     st(c + i, x);
@@ -410,7 +412,8 @@ extern "C" int llmx_gemm_skinny_normed_ok(int x_rows, int K) {
 extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                                 int n_groups, int max_active, const int* active, const int* n_active, const int* group_offsets,
                                 const int* list, int a_div, long w_group_stride, int up_offset, const float* X, const float* norm_w,
-                                float norm_eps, int x_rows, int act, const float* act_params, hipStream_t stream) {
+                                float norm_eps, int x_rows, int act, const float* act_params, int glu_kind, float glu_limit,
+                                const float* glu_row_scale, const float* glu_row_gate, int glu_row_gate_ld, hipStream_t stream) {
     if (N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
@@ -418,7 +421,9 @@ extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dty
     if (grouped && max_active <= 0) return 0;
     if (X && (!norm_w || epi == SK_ADD || !llmx_gemm_skinny_normed_ok(x_rows, K) || (!grouped && x_rows != M))) return -2;
     SkinnyArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, active, n_active, group_offsets, list, a_div > 0 ? a_div : 1,
-                 w_group_stride, up_offset, X, norm_w, norm_eps, x_rows, epi == SK_STORE ? act : LLMX_ACT_NONE, act_params};
+                 w_group_stride, up_offset, X, norm_w, norm_eps, x_rows, epi == SK_STORE ? act : LLMX_ACT_NONE, act_params,
+                 GluArgs{epi == SK_SWIGLU ? glu_kind : LLMX_GLU_SILU, glu_limit, epi == SK_SWIGLU ? glu_row_scale : nullptr,
+                         epi == SK_SWIGLU ? glu_row_gate : nullptr, glu_row_gate_ld}};
     if (act != LLMX_ACT_NONE && (epi != SK_STORE || !act_params)) return -2;
     dim3 grid((N + 15) / 16, grouped ? max_active : 1, 1);
     int mt = 1;

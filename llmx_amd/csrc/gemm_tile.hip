@@ -87,6 +87,7 @@ struct TileArgs {
     int run_tiles;          // dense lean form, > 0: workgroup z multiplies only K's run z (this many 64-wide tiles) and stores its sums at C + z * M * ldc
     int act;                // TL_STORE: an activation applied to what is stored (LLMX_ACT_*; a launch of runs' sums leaves it to the kernel that adds them)
     const float* act_params;
+    GluArgs glu;            // TL_SWIGLU: the gated unit and its per-row values
 };
 
 // Whether the groups' rows fill tiles of 128 rows well enough: the tiles hold at most 1.6 times the rows (measured on
@@ -436,14 +437,12 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         if (rc < 0) continue;
         TC* crow = (TC*)g.C + (size_t)rc * g.ldc + (g.run_tiles > 0 ? (size_t)blockIdx.z * g.M * g.ldc : 0);
         if (EPI == TL_SWIGLU) {
+            const GluRow glu(g.glu, rc);
 #pragma unroll
             for (int f = 0; f < 2; ++f) {
                 float v[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float gt = acc[f][t][i], u = acc[f + 2][t][i];
-                    v[i] = (gt / (1.0f + expf(-gt))) * u;
-                }
+                for (int i = 0; i < 4; ++i) v[i] = glu(acc[f][t][i], acc[f + 2][t][i]);
                 store_quad<false>(crow, n0 + 32 * wn + 16 * f + fq, g.N, rows_aligned, v);
             }
         } else {
@@ -708,14 +707,12 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
         if (rc < 0) continue;
         TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
         if (EPI == TL_SWIGLU) {
+            const GluRow glu(g.glu, rc);
 #pragma unroll
             for (int f = 0; f < 2; ++f) {
                 float v[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float gt = acc[f][q][i], u = acc[f + 2][q][i];
-                    v[i] = (gt / (1.0f + expf(-gt))) * u;
-                }
+                for (int i = 0; i < 4; ++i) v[i] = glu(acc[f][q][i], acc[f + 2][q][i]);
                 store_quad<false>(crow, n0 + 32 * wn + 16 * f + fq, g.N, rows_aligned, v);
             }
         } else {
@@ -844,7 +841,8 @@ extern "C" long llmx_gemm_tile_runs_scratch(int M, int N, int K, int epi, int ks
 
 extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                               int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,
-                              int up_offset, const int* tile_stats, float* runs_scratch, int act, const float* act_params, hipStream_t stream) {
+                              int up_offset, const int* tile_stats, float* runs_scratch, int act, const float* act_params, int glu_kind,
+                              float glu_limit, const float* glu_row_scale, const float* glu_row_gate, int glu_row_gate_ld, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
@@ -852,7 +850,9 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
     const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0) && llmx_gemm_tile_offsets_fit(M, N, K, lda, epi, n_groups, a_div, up_offset);
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
-               w_group_stride, up_offset, 0, ks, 64, nullptr, 0, 0, epi == TL_STORE ? act : LLMX_ACT_NONE, act_params};
+               w_group_stride, up_offset, 0, ks, 64, nullptr, 0, 0, epi == TL_STORE ? act : LLMX_ACT_NONE, act_params,
+               GluArgs{epi == TL_SWIGLU ? glu_kind : LLMX_GLU_SILU, glu_limit, epi == TL_SWIGLU ? glu_row_scale : nullptr,
+                       epi == TL_SWIGLU ? glu_row_gate : nullptr, glu_row_gate_ld}};
     if (act != LLMX_ACT_NONE && (epi != TL_STORE || !act_params)) return -2;
     auto launch = [&](int form, int tiles_y) -> int {
         g.bm = form_rows(form);

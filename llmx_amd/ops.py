@@ -72,7 +72,7 @@ def _declare(h) -> None:
         "llmx_fill_random": [P, I, L, ctypes.c_ulonglong, I, F, F, P],
         "llmx_read_probe": [P, L, P, P],
         "llmx_attention_partial_pad": [],
-        "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, P],
+        "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, I, F, P, P, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P],
         "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P, I, P],
@@ -94,12 +94,12 @@ def _declare(h) -> None:
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
-        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P, P, F, I, I, P, P],
+        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P, P, F, I, I, P, I, F, P, P, I, P],
         "llmx_gemm_skinny_normed_ok": [I, I],
         "llmx_gemm_skinny_f32_normed_ok": [I, I],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P, F, P],
-        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P, I, P, P],
+        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P, I, P, I, F, P, P, I, P],
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P, I, P],
@@ -255,6 +255,15 @@ class Glu:
     @property
     def plain(self) -> bool:
         return self.kind == GLU_SILU and self.row_scale is None and self.row_gate is None
+
+    def args(self, rows: int):
+        """The five values the product kernels take, checked against the `rows` rows of c."""
+        gate_at, gate_ld = _rows_view(self.row_gate, "row_gate", rows, 1) if self.row_gate is not None else (0, 0)
+        return self.kind, self.limit, _dev(self.row_scale, "row_scale", torch.float32, (rows,)), gate_at, gate_ld
+
+
+_NO_GLU = (0, 0.0, 0, 0, 0)
+GLU_IN_EPILOGUE = True      # False: a product with another unit than silu(gate) * up stores its pre-activations and the unit's own kernel follows
 
 
 def act_glu(pre: torch.Tensor, glu: Glu, out: torch.Tensor) -> None:
@@ -757,7 +766,7 @@ def _glu_apart(glu: Optional["Glu"], epilogue: int) -> bool:
         return False
     if epilogue != EPI_SWIGLU:
         raise KernelError("a gated unit goes with the gated epilogue")
-    return not glu.plain
+    return not glu.plain and not GLU_IN_EPILOGUE
 
 
 def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False, scratch=None, act=None,
@@ -777,6 +786,7 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
         gemm(a, w, pre, EPI_STORE, force_generic, scratch)
         act_glu(pre, glu, c)
         return
+    glu_args = glu.args(M) if glu is not None and not glu.plain else _NO_GLU
     act_args = (0, 0)
     if act is not None:
         if epilogue != EPI_STORE or act[0] != ACT_XIELU:
@@ -789,7 +799,7 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
         if not gemm_can_norm_rows(M, w, c.dtype, epilogue):
             raise KernelError("gemm: normed rows are not taken for this product")
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), *act_args, _stream()),
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), *act_args, *glu_args, _stream()),
                "gemm_skinny (normed rows)")
         return
     # a product wide enough to fill the chip with tiles (the LM head) streams its weights faster through the tiled kernel
@@ -806,16 +816,16 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
         skinny = False
     if not force_generic and skinny and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, *act_args, _stream()),
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, *act_args, *glu_args, _stream()),
                "gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         runs = scratch("gemm_tile.runs", (runs_apart,), torch.float32) if runs_apart else None
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                    ks, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _dev(runs, "runs"), *act_args, _stream()), "gemm_tile")
+                                    ks, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _dev(runs, "runs"), *act_args, *glu_args, _stream()), "gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
-                                   M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *act_args, _stream()), "gemm")
+                                   M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *act_args, *glu_args, _stream()), "gemm")
 
 
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
@@ -840,6 +850,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
     if a.shape[1] != K or c.shape[1] != N:
         raise KernelError(f"grouped_gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
     n_pairs = pairs.shape[0]
+    glu_args = glu.args(c.shape[0]) if glu is not None and not glu.plain else _NO_GLU
     if c.shape[0] < n_pairs or a.shape[0] * a_div < n_pairs:
         raise KernelError("grouped_gemm: more pairs than rows")
     if token_rows is None:
@@ -850,7 +861,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *a.args(), 0, 0, _stream()),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *a.args(), 0, 0, *glu_args, _stream()),
                "grouped_gemm_skinny (normed rows)")
         return
     if (not force_generic and active is not None and n_active is not None and _skinny_ok(a, w, c, epilogue)
@@ -858,19 +869,19 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, 0, 0, _stream()),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, 0, 0, *glu_args, _stream()),
                "grouped_gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                     _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 64, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                     _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0,
-                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, 0, 0, _stream()),
+                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, 0, 0, *glu_args, _stream()),
                "grouped_gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    n_pairs, N, K, K, K, N, epilogue, G, _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, 0, 0, _stream()),
+                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, 0, 0, *glu_args, _stream()),
            "grouped_gemm")
 
 

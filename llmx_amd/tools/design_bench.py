@@ -4,6 +4,11 @@
 gated linear attention, the delta rule alone; routed SwiGLU experts) and a MiniMax-M3 with the same width, layers, heads,
 head width and experts.
 
+`python bench.py --design givozen` does the same for a Givozen (a dense layer with the polynomial activation, then layers of
+routed clamped-unit experts with a shared expert, two of them run twice; attention with biases, a temperature and a gate
+a head) and a MiniMax-M3 with as many layers as the Givozen has layer runs and the same width, heads, head width, experts,
+picks and expert width.  A repeated layer's weights count each time they run.
+
 `python bench.py --design nenotar` measures, at sizes that resemble a real model's layers, a Nenotar (latent attention
 and minGRU layers in turn, each with a dense xIELU feed-forward and a per-layer token input) and a MiniMax-M3 of the
 same width, layers, heads and vocabulary whose routed experts hold the same active weights a token: one 2,048-token
@@ -85,6 +90,57 @@ def bonerax_closest(width, layers, heads, kv_heads, window, rec_heads, experts, 
                            max_position_embeddings=2 * CONTEXT)
 
 
+# name -> (width, layers, heads, kv heads, dense ff, experts, picks, expert ff, shared ff, loop (start, stop, times), vocab)
+GIVOZEN_SIZES = {
+    "w2048": (2048, 6, 16, 4, 8192, 8, 2, 2048, 2048, (1, 3, 2), 32768),
+    "w4096": (4096, 3, 32, 8, 16384, 8, 2, 4096, 4096, (1, 2, 2), 32768),
+    "w256": (256, 3, 2, 1, 768, 4, 2, 128, 64, (1, 2, 2), 1024),
+}
+
+
+def givozen_config(width, layers, heads, kv_heads, dense_ff, experts, top, ff, shared_ff, loop, vocab):
+    from llmx_amd.config.givozen import AttentionConfig, GivozenConfig, LayerConfig, LoopConfig, MLPConfig, SharedExpertConfig, WavelengthScaling
+    mixer = AttentionConfig(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, rot_base=1e6, rot_dims=64,
+                            rot_scaling=WavelengthScaling(8.0, 1.0, 4.0, 8192.0))
+    moe = MLPConfig("moe", ff, limit=7.0, experts=experts, top=top, shared=SharedExpertConfig(shared_ff, 7.0))
+    kinds = [LayerConfig("attention", mixer, MLPConfig("dense", dense_ff) if i == 0 else moe) for i in range(layers)]
+    return GivozenConfig(vocab=vocab, width=width, norm_eps=1e-6, layers=tuple(kinds), loop=LoopConfig(*loop))
+
+
+def givozen_closest(width, layers, heads, kv_heads, dense_ff, experts, top, ff, shared_ff, loop, vocab):
+    """MiniMax-M3 with a layer for every layer run of the Givozen, the same width, heads, head width, experts, picks and
+    expert width."""
+    from llmx_amd import MiniMaxM3Config
+    runs = layers + (loop[1] - loop[0]) * (loop[2] - 1)
+    return MiniMaxM3Config(vocab_size=vocab, hidden_size=width, num_hidden_layers=runs, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                           head_dim=128, rotary_dim=64, rope_theta=1e6, rms_norm_eps=1e-6, num_local_experts=experts, num_experts_per_tok=top,
+                           intermediate_size=ff, routed_scaling_factor=1.0, norm_topk_prob=True, tie_word_embeddings=False,
+                           max_position_embeddings=2 * CONTEXT)
+
+
+def givozen_work(cfg, rows: int):
+    """(weights a step of `rows` rows multiplies a row by, weights it must read), both in elements, summed over the layer
+    runs (a repeated layer counts each time it runs); of routed experts a row uses `top` and a step reads at most rows x top."""
+    used = read = 0.0
+    for i, _, _ in cfg.passes():
+        layer = cfg.layers[i]
+        a = layer.mixer
+        attention = cfg.width * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim) + a.heads) + a.heads * a.vdim * cfg.width
+        used += attention
+        read += attention
+        mlp = layer.mlp
+        if mlp is None:
+            continue
+        if mlp.kind == "dense":
+            used += 2 * cfg.width * mlp.ff
+            read += 2 * cfg.width * mlp.ff
+            continue
+        fixed = cfg.width * mlp.experts + (3 * cfg.width * mlp.shared.ff + cfg.width if mlp.shared else 0)
+        used += fixed + mlp.top * 3 * cfg.width * mlp.ff
+        read += fixed + min(mlp.experts, rows * mlp.top) * 3 * cfg.width * mlp.ff
+    return used, read
+
+
 def _layer_mixers(layer):
     """(windowed attention or None, [recurrences as (heads, dim, vdim, delta?)]) of a Bonerax layer."""
     m = layer.mixer
@@ -129,6 +185,9 @@ def prompt_flops(engine, T) -> float:
         expert = 3 * cfg.hidden_size * cfg.intermediate_size
         dense -= 2.0 * T * cfg.num_hidden_layers * (cfg.num_local_experts - cfg.num_experts_per_tok) * expert
         attn = cfg.num_hidden_layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * T * (T + 1) / 2
+    elif cfg.architecture == "Givozen":
+        dense = 2.0 * T * givozen_work(cfg, T)[0] + 2.0 * vocab * engine.spec.hidden_size
+        attn = sum(2.0 * cfg.layers[i].mixer.heads * (cfg.layers[i].mixer.dim + cfg.layers[i].mixer.vdim) * T * (T + 1) / 2 for i, _, _ in cfg.passes())
     elif cfg.architecture == "Bonerax":
         attn = 0.0
         for layer in cfg.layers:
@@ -213,6 +272,8 @@ def measure(engine, torch, steps, warmup):
         side = getattr(cfg, "token_side_dim", None) or 0
         need -= 2 * vocab * side * (len(cfg.layers) if side else 0)     # of the token table a step reads its rows only
         need -= 2 * vocab * engine.spec.hidden_size                     # and of the embedding
+        if cfg.architecture == "Givozen":       # weights by layer run; the head is the embedding's table, read whole
+            need = 2 * (givozen_work(cfg, batch)[1] + vocab * engine.spec.hidden_size) + batch * cache_bytes_read(engine, CONTEXT - steps / 2)
         rec.update({f"decode_b{batch}_tok_s": round(batch / dt, 2), f"decode_b{batch}_ms": round(dt * 1e3, 4),
                     f"decode_b{batch}_gb": round(need / 1e9, 3), f"decode_b{batch}_frac": round(need / dt / 1e9 / HBM_PEAK_GBS, 4)})
     return rec
@@ -221,6 +282,7 @@ def measure(engine, torch, steps, warmup):
 DESIGNS = {
     "nenotar": ("Nenotar", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", SIZES, nenotar_config, closest_config),
     "bonerax": ("Bonerax", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", BONERAX_SIZES, bonerax_config, bonerax_closest),
+    "givozen": ("Givozen", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", GIVOZEN_SIZES, givozen_config, givozen_closest),
 }
 
 

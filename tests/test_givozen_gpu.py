@@ -98,14 +98,25 @@ def test_gated_unit_with_a_factor_on_its_input_and_a_switch(kind):
         close(out, plain_g * plain.sigmoid(plain_g) * plain_u, 3e-6)
 
 
+@pytest.fixture(params=[True, False], ids=["in the epilogue", "a kernel of its own"])
+def unit_in_epilogue(request):
+    o = ops()
+    before = o.GLU_IN_EPILOGUE
+    o.GLU_IN_EPILOGUE = request.param
+    yield request.param
+    o.GLU_IN_EPILOGUE = before
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
-def test_products_with_a_gated_unit_dense_and_grouped(dtype):
+def test_products_with_a_gated_unit_dense_and_grouped(dtype, unit_in_epilogue):
     """gemm and grouped_gemm with a gated unit (clamped, a factor on each row's input, a switch on its result) against the
-    plain expert, at a few row counts (the weight-streaming and the tiled products) and widths."""
+    plain expert, at a few row counts (the weight-streaming and the tiled products) and widths; the unit in the products'
+    epilogue, and as a kernel of its own behind a storing product."""
     rng = np.random.default_rng(11)
     o = ops()
+    o.take_launches()
     tol = 2e-5 if dtype == torch.float32 else 2.5e-2
-    for rows, E, F in ((1, 64, 32), (9, 128, 48), (70, 64, 96)):
+    for rows, E, F in ((1, 64, 32), (9, 128, 48), (70, 64, 96), (300, 128, 256)):
         h = rng.normal(size=(rows, E))
         wg, wu = rng.normal(size=(F, E)) * 0.2, rng.normal(size=(F, E)) * 0.2
         w = {"e.gate": wg, "e.up": wu, "e.down": np.eye(F)}
@@ -135,6 +146,7 @@ def test_products_with_a_gated_unit_dense_and_grouped(dtype):
                 we = {"x.gate": wgur[e, :F], "x.up": wgur[e, F:], "x.down": np.eye(F)}
                 want = plain.clamped_glu_expert(np.float32(score[t, j]) * hr[t:t + 1], we, "x.", 1.3)[0]
                 close(act[t * k + j].float(), want, tol, f"grouped row {t} slot {j}")
+    assert bool(o.take_launches().get("act.glu")) == (not unit_in_epilogue)
 
 
 def test_gate_a_head_pass_vector_offset_norm_and_unit_combine():
@@ -435,6 +447,7 @@ def test_which_kernels_a_serving_step_takes():
                 seen[name] = seen.get(name, 0) + count
         for name in ("head_norm_rope_kvwrite", "gate_heads", "act.polynorm", "add_rows_vector", "rmsnorm_add", "rmsnorm", "moe_combine"):
             assert seen.get(name), f"{dtype}: no launch of {name} ({sorted(seen)})"
+        assert "act.glu" not in seen          # the experts' unit runs in their first product's epilogue
         assert seen["add_rows_vector"] == 2 * 3 and seen["gate_heads"] == 2 * 8           # three passes, eight layer runs, two steps
         if dtype == "bfloat16":
             assert not any(n.startswith(("gemm_generic", "attention.generic")) for n in seen), sorted(seen)
