@@ -67,22 +67,49 @@ extern "C" int llmx_scale_add(float* x, const float* y1, const float* s1, const 
 }
 
 // ---------------------------------------------------------------------------
-// x[t,:] += y[t,:] * (r * w[:]), r = 1 / sqrt(mean(y[t,:]^2) + eps): a result joined after its own RMS norm.
-__global__ void __launch_bounds__(256) rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
-                                                        float eps, int n) {
-    __shared__ float scratch[4];
+// x[t,:] += y[t,:] * (r * w[:]), r = 1 / sqrt(mean(y[t,:]^2) + eps): a result joined after its own RMS norm.  One block of
+// 1,024 threads a row; the sum as the norm kernels form it (a thread's elements in stride order with fmaf, a butterfly a
+// wave, the waves in order), which is also the first sum of rmsnorm_add_norm_kernel: both give x the same bits.  Rows of at
+// most 8,192 values are kept in registers, all loads asked for before the sum.
+#define ADD_THREADS 1024
+#define ADD_KEPT 8
+__global__ void __launch_bounds__(ADD_THREADS) rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
+                                                                 float eps, int n) {
+    __shared__ float scratch[ADD_THREADS / 64];
     const int r = blockIdx.x;
     const float* row = y + (size_t)r * n;
-    const float s = block_sum<4>(strided_squares<256>(row, n), scratch);
-    const float scale = 1.0f / sqrtf(s / (float)n + eps);
     float* out = x + (size_t)r * n;
-    for (int i = threadIdx.x; i < n; i += 256) out[i] = out[i] + row[i] * (scale * w[i]);
+    if (n <= ADD_THREADS * ADD_KEPT) {
+        float vx[ADD_KEPT], vy[ADD_KEPT], wj[ADD_KEPT];
+#pragma unroll
+        for (int e = 0; e < ADD_KEPT; ++e) {
+            const int i = threadIdx.x + e * ADD_THREADS;
+            const bool in = i < n;
+            vy[e] = in ? row[i] : 0.0f;
+            vx[e] = in ? out[i] : 0.0f;
+            wj[e] = in ? w[i] : 0.0f;
+        }
+        float sq = 0.0f;
+#pragma unroll
+        for (int e = 0; e < ADD_KEPT; ++e) sq = fmaf(vy[e], vy[e], sq);
+        const float scale = 1.0f / sqrtf(block_sum<ADD_THREADS / 64>(sq, scratch) / (float)n + eps);
+#pragma unroll
+        for (int e = 0; e < ADD_KEPT; ++e) {
+            const int i = threadIdx.x + e * ADD_THREADS;
+            if (i < n) out[i] = vx[e] + vy[e] * (scale * wj[e]);
+        }
+        return;
+    }
+    float sq = 0.0f;
+    for (int i = threadIdx.x; i < n; i += ADD_THREADS) sq = fmaf(row[i], row[i], sq);
+    const float scale = 1.0f / sqrtf(block_sum<ADD_THREADS / 64>(sq, scratch) / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += ADD_THREADS) out[i] = out[i] + row[i] * (scale * w[i]);
 }
 
 extern "C" int llmx_rmsnorm_add(float* x, const float* y, const float* w, float eps, int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
     llmx_note_launch(LK_RMSNORM_ADD);
-    hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(rows), dim3(256), 0, stream, x, y, w, eps, n);
+    hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(rows), dim3(ADD_THREADS), 0, stream, x, y, w, eps, n);
     return LLMX_CHECK_LAUNCH();
 }
 
@@ -239,5 +266,87 @@ extern "C" int llmx_act_glu(const float* pre, int ld, const float* row_scale, co
         hipLaunchKernelGGL(glu_kernel<float>, grid, dim3(256), 0, stream, pre, ld, row_scale, row_gate, row_gate_ld, kind, limit, (float*)out, n, total);
     else
         hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, dim3(256), 0, stream, pre, ld, row_scale, row_gate, row_gate_ld, kind, limit, (bf16_t*)out, n, total);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// A result joined after its own RMS norm, and the next sublayer's norm of the new row, in one pass:
+// x[t,:] += y[t,:] * (r_y * w_join[:]); h[t,:] = x[t,:] * (r_x * w_next[:]), r_v = 1 / sqrt(mean(v^2) + eps_v).
+// One block of 1,024 threads a row; rows of at most 8,192 values stay in registers between the two sums (every load is
+// asked for before the first sum), longer rows are read again.  Each sum: a thread's elements in stride order with fmaf, a
+// butterfly a wave, the waves in order.  h is stored in the activation type and/or as float32.
+#define JOIN_THREADS 1024
+#define JOIN_KEPT 8
+template <typename TO>
+__global__ void __launch_bounds__(JOIN_THREADS) rmsnorm_add_norm_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                      const float* __restrict__ w_join, float eps_join,
+                                                                      const float* __restrict__ w_next, float eps_next, TO* __restrict__ out,
+                                                                      float* __restrict__ out32, int n) {
+    __shared__ float scratch[JOIN_THREADS / 64];
+    const int r = blockIdx.x;
+    float* xr = x + (size_t)r * n;
+    const float* yr = y + (size_t)r * n;
+    if (n <= JOIN_THREADS * JOIN_KEPT) {
+        float vx[JOIN_KEPT], vy[JOIN_KEPT], wj[JOIN_KEPT], wn[JOIN_KEPT];
+#pragma unroll
+        for (int e = 0; e < JOIN_KEPT; ++e) {
+            const int i = threadIdx.x + e * JOIN_THREADS;
+            const bool in = i < n;
+            vy[e] = in ? yr[i] : 0.0f;
+            vx[e] = in ? xr[i] : 0.0f;
+            wj[e] = in ? w_join[i] : 0.0f;
+            wn[e] = in ? w_next[i] : 0.0f;
+        }
+        float sq = 0.0f;
+#pragma unroll
+        for (int e = 0; e < JOIN_KEPT; ++e) sq = fmaf(vy[e], vy[e], sq);
+        const float scale_y = 1.0f / sqrtf(block_sum<JOIN_THREADS / 64>(sq, scratch) / (float)n + eps_join);
+        sq = 0.0f;
+#pragma unroll
+        for (int e = 0; e < JOIN_KEPT; ++e) {
+            vx[e] = vx[e] + vy[e] * (scale_y * wj[e]);      // an element past the end stays 0
+            sq = fmaf(vx[e], vx[e], sq);
+        }
+        const float scale_x = 1.0f / sqrtf(block_sum<JOIN_THREADS / 64>(sq, scratch) / (float)n + eps_next);
+#pragma unroll
+        for (int e = 0; e < JOIN_KEPT; ++e) {
+            const int i = threadIdx.x + e * JOIN_THREADS;
+            if (i < n) {
+                xr[i] = vx[e];
+                const float h = vx[e] * (scale_x * wn[e]);
+                if (out) st(out + (size_t)r * n + i, h);
+                if (out32) out32[(size_t)r * n + i] = h;
+            }
+        }
+        return;
+    }
+    float sq = 0.0f;
+    for (int i = threadIdx.x; i < n; i += JOIN_THREADS) sq = fmaf(yr[i], yr[i], sq);
+    const float scale_y = 1.0f / sqrtf(block_sum<JOIN_THREADS / 64>(sq, scratch) / (float)n + eps_join);
+    sq = 0.0f;
+    for (int i = threadIdx.x; i < n; i += JOIN_THREADS) {      // a thread reads back only what it wrote
+        const float v = xr[i] + yr[i] * (scale_y * w_join[i]);
+        xr[i] = v;
+        sq = fmaf(v, v, sq);
+    }
+    const float scale_x = 1.0f / sqrtf(block_sum<JOIN_THREADS / 64>(sq, scratch) / (float)n + eps_next);
+    for (int i = threadIdx.x; i < n; i += JOIN_THREADS) {
+        const float h = xr[i] * (scale_x * w_next[i]);
+        if (out) st(out + (size_t)r * n + i, h);
+        if (out32) out32[(size_t)r * n + i] = h;
+    }
+}
+
+extern "C" int llmx_rmsnorm_add_norm(float* x, const float* y, const float* w_join, float eps_join, const float* w_next, float eps_next,
+                                     void* out, int out_dtype, float* out32, int rows, int n, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (!w_join || !w_next || (!out && !out32)) return -2;
+    llmx_note_launch(LK_RMSNORM_ADD_NORM);
+    if (out_dtype == LLMX_F32)
+        hipLaunchKernelGGL(rmsnorm_add_norm_kernel<float>, dim3(rows), dim3(JOIN_THREADS), 0, stream, x, y, w_join, eps_join, w_next, eps_next,
+                           (float*)out, out32, n);
+    else
+        hipLaunchKernelGGL(rmsnorm_add_norm_kernel<bf16_t>, dim3(rows), dim3(JOIN_THREADS), 0, stream, x, y, w_join, eps_join, w_next, eps_next,
+                           (bf16_t*)out, out32, n);
     return LLMX_CHECK_LAUNCH();
 }

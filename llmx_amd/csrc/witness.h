@@ -77,7 +77,8 @@
     X(ADD_ROWS_VECTOR, "add_rows_vector")                                                                                 \
     X(ACT_POLYNORM, "act.polynorm")                                                                                       \
     X(ACT_GLU, "act.glu")                                                                                                 \
-    X(GATE_HEADS, "gate_heads")
+    X(GATE_HEADS, "gate_heads")                                                                                           \
+    X(RMSNORM_ADD_NORM, "rmsnorm_add_norm")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

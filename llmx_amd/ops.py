@@ -77,6 +77,7 @@ def _declare(h) -> None:
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P],
         "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P, I, P],
         "llmx_gate_heads": [P, I, P, I, I, I, I, P],
+        "llmx_rmsnorm_add_norm": [P, P, P, F, P, F, P, I, P, I, I, P],
         "llmx_add_rows_vector": [P, P, P, I, I, P],
         "llmx_act_polynorm": [P, P, F, P, I, I, I, P],
         "llmx_act_glu": [P, I, P, P, I, I, F, P, I, I, I, P],
@@ -275,6 +276,19 @@ def act_glu(pre: torch.Tensor, glu: Glu, out: torch.Tensor) -> None:
     gate_at, gate_ld = _rows_view(glu.row_gate, "row_gate", P, 1) if glu.row_gate is not None else (0, 0)
     _check(lib().llmx_act_glu(_dev(pre, "pre", torch.float32), pre.shape[1], _dev(glu.row_scale, "row_scale", torch.float32, (P,)),
                               gate_at, gate_ld, glu.kind, glu.limit, _dev(out, "out"), _code(out.dtype), P, n, _stream()), "act_glu")
+
+
+def rmsnorm_add_norm(x: torch.Tensor, y: torch.Tensor, w_join: torch.Tensor, eps_join: float, w_next: torch.Tensor, eps_next: float,
+                     out: Optional[torch.Tensor], out32: Optional[torch.Tensor] = None) -> None:
+    """x += RMSNorm(y) * w_join, then out / out32 = RMSNorm(x) * w_next of the new rows: a sublayer's normed result joined
+    into the residual and the next sublayer's norm in one launch.  x, y float32 [T, n]; out in its own type, out32 float32."""
+    rows, n = x.shape
+    if out is None and out32 is None:
+        raise KernelError("rmsnorm_add_norm needs an output")
+    _check(lib().llmx_rmsnorm_add_norm(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, (rows, n)), _dev(w_join, "w_join", torch.float32, (n,)),
+                                       float(eps_join), _dev(w_next, "w_next", torch.float32, (n,)), float(eps_next),
+                                       _dev(out, "out", shape=(rows, n)), _code(out.dtype) if out is not None else F32,
+                                       _dev(out32, "out32", torch.float32, (rows, n)), rows, n, _stream()), "rmsnorm_add_norm")
 
 
 def act_xielu(z: torch.Tensor, pq: torch.Tensor, out: torch.Tensor) -> None:

@@ -201,6 +201,9 @@ class SandwichBlock:
         for n in (self.mixer_post, self.ffn_post):
             if n is not None and not hasattr(n, "add_into"):
                 raise ValueError(f"sandwich block: the norm {n.kind!r} cannot join a result into the residual (no add_into)")
+        # RMS norms on both sides of the join before the feed-forward: one launch joins the mixer's result and norms the new rows
+        self._join_then_norm = (self.ffn is not None and isinstance(self.mixer_post, RMSNorm) and isinstance(self.ffn_norm, RMSNorm)
+                                and self.mixer_post.width == self.ffn_norm.width)
 
     def parts(self):
         return [p for p in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post) if p is not None]
@@ -210,11 +213,18 @@ class SandwichBlock:
         y = step.buf("block.y", (T, E), torch.float32)
         h, h32 = PreNormBlock.normed(step, self.mixer_norm, self.mixer, x)
         self.mixer.forward(step, h, y, False, cache, h32)
-        self.mixer_post.add_into(step, x, y)
-        if self.ffn is not None:
+        if self.ffn is None:
+            self.mixer_post.add_into(step, x, y)
+            return
+        if self._join_then_norm and not (self.ffn_norm.deferred(x) is not None and self.ffn.takes_deferred_norm(step)):
+            h = step.buf("block.h", (T, E), step.act_dtype)
+            h32 = step.buf("block.h32", (T, E), torch.float32) if self.ffn.wants_f32_input else None
+            self.mixer_post.add_into_then_norm(step, x, y, self.ffn_norm, h, h32)
+        else:
+            self.mixer_post.add_into(step, x, y)
             h, h32 = PreNormBlock.normed(step, self.ffn_norm, self.ffn, x)
-            self.ffn.forward(step, h, y, False, h32)
-            self.ffn_post.add_into(step, x, y)
+        self.ffn.forward(step, h, y, False, h32)
+        self.ffn_post.add_into(step, x, y)
 
 
 register("block", "prenorm", PreNormBlock)

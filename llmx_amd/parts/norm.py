@@ -65,6 +65,10 @@ class RMSNorm(Norm):
         if copy is not None:
             ops.cast_rows(x, copy)
 
+    def add_into_then_norm(self, step, x, y, then: "RMSNorm", out, out32=None):
+        """x += norm(y); out / out32 = then(x): the join and the next sublayer's norm in one launch."""
+        ops.rmsnorm_add_norm(x, y, self.weight, self.eps, then.weight, then.eps, out, out32)
+
 
 class LayerNorm(Norm):
     """params: width, eps; tensor (the name's last part, "weight" by default; "" when the prefix is the whole name).

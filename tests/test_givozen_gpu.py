@@ -186,6 +186,27 @@ def test_gate_a_head_pass_vector_offset_norm_and_unit_combine():
     close(acc, x + y.reshape(T, k, E).sum(1), 2e-6)
 
 
+@pytest.mark.parametrize("rows,n", [(1, 8), (5, 54), (3, 1030), (2, 8200)])
+def test_join_and_next_norm_in_one_launch(rows, n):
+    """x += N_join(y); h = N_next(x) as one kernel: the plain functions' values, and bit for bit the join kernel followed by
+    the norm kernel (a block may use either way for the same place in the model)."""
+    rng = np.random.default_rng(n + rows)
+    o = ops()
+    x, y = rng.normal(size=(rows, n)) * 3, rng.normal(size=(rows, n)) * 0.5
+    wj, wn = 1.0 + rng.normal(size=n) * 0.2, 1.0 + rng.normal(size=n) * 0.2
+    xd, h16, h32 = dev(x), torch.empty(rows, n, device="cuda", dtype=torch.bfloat16), torch.empty(rows, n, device="cuda")
+    o.rmsnorm_add_norm(xd, dev(y), dev(wj), 1e-5, dev(wn), 1e-3, h16, h32)
+    f32 = lambda a: np.asarray(a, dtype=np.float32).astype(np.float64)
+    want_x = f32(x) + plain.rms_unit(f32(y), 1e-5) * f32(wj)
+    close(xd, want_x, 2e-6, "the joined rows")
+    close(h32, plain.rms_unit(want_x, 1e-3) * f32(wn), 3e-6, "their norm")
+    assert torch.equal(h16, h32.to(torch.bfloat16))
+    x2, g32 = dev(x), torch.empty(rows, n, device="cuda")
+    o.rmsnorm_add(x2, dev(y), dev(wj), 1e-5)
+    o.rmsnorm(x2, dev(wn), 1e-3, None, g32)
+    assert torch.equal(x2, xd) and torch.equal(g32, h32)
+
+
 def _attention_case(dtype, H, G, D, VD, R, scaling, page, length, sharp=None, decode_from=None, scale=0.3):
     """One attention part alone through its kernels (the step with biases and a temperature a head, the attention over
     shuffled pages, the gate a head) against the plain mixer.  sharp = (row, key): the row's query is made to fit that key
@@ -445,10 +466,12 @@ def test_which_kernels_a_serving_step_takes():
             engine.step([entry])
             for name, count in o.take_launches().items():
                 seen[name] = seen.get(name, 0) + count
-        for name in ("head_norm_rope_kvwrite", "gate_heads", "act.polynorm", "add_rows_vector", "rmsnorm_add", "rmsnorm", "moe_combine"):
+        for name in ("head_norm_rope_kvwrite", "gate_heads", "act.polynorm", "add_rows_vector", "rmsnorm_add", "rmsnorm_add_norm", "rmsnorm",
+                     "moe_combine"):
             assert seen.get(name), f"{dtype}: no launch of {name} ({sorted(seen)})"
         assert "act.glu" not in seen          # the experts' unit runs in their first product's epilogue
         assert seen["add_rows_vector"] == 2 * 3 and seen["gate_heads"] == 2 * 8           # three passes, eight layer runs, two steps
+        assert seen["rmsnorm_add_norm"] == 2 * 7 and seen["rmsnorm_add"] == 2 * 8        # seven runs have a feed-forward; its join and the last layer's
         if dtype == "bfloat16":
             assert not any(n.startswith(("gemm_generic", "attention.generic")) for n in seen), sorted(seen)
             assert any(n.startswith("attention.") for n in seen) and any(n.startswith("gemm_skinny") or n.startswith("gemm_tile") for n in seen)
