@@ -399,6 +399,8 @@ struct AttnArgs {
     float scale;
     int n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
     int v_dim;   // width of a value head (the output's too); keys and queries have head_dim
+    const float* gate;  // null, or a float32 logit a (row, head), row stride gate_ld: the output is multiplied by its sigmoid
+    int gate_ld;
 };
 
 #define ATT_MAX_D 256
@@ -465,19 +467,22 @@ __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a)
         __syncthreads();
     }
     T* out = (T*)a.out + ((size_t)t * a.n_heads + h) * VD;
+    const float factor = a.gate ? sigmoid_f(a.gate[(size_t)t * a.gate_ld + h]) : 1.0f;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
-        if (d < VD) st(out + d, acc[i] / l);
+        if (d < VD) st(out + d, acc[i] / l * factor);
     }
 }
 
 extern "C" int llmx_paged_attention_generic(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
                                             const int* tables, void* out, int dtype, float scale, int rows, int n_heads, int n_kv_heads,
-                                            int head_dim, int page_tokens, int max_blocks, int window, int v_dim, hipStream_t stream) {
+                                            int head_dim, int page_tokens, int max_blocks, int window, int v_dim, const float* gate, int gate_ld,
+                                            hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (head_dim > ATT_MAX_D || v_dim > ATT_MAX_D || v_dim < 1 || n_heads % n_kv_heads) return -2;
-    AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window, v_dim};
+    if (head_dim > ATT_MAX_D || v_dim > ATT_MAX_D || v_dim < 1 || n_heads % n_kv_heads || (gate && gate_ld < n_heads)) return -2;
+    AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window, v_dim,
+               gate, gate_ld};
     llmx_note_launch(LK_ATTENTION_GENERIC);
     if (dtype == LLMX_F32)
         hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(rows, n_heads), dim3(64), 0, stream, a);

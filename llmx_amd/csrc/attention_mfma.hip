@@ -141,14 +141,19 @@ __device__ __forceinline__ uint32_t segment_mask(int seg0, int g, bool col_ok, i
     return ok;
 }
 
-// the column's output row: lane holds dims 16dt + 4g + i
+// The factor on the output of (row t, head h): sigmoid of the head's gate logit (float32, row stride ldg), or 1 without a gate.
+__device__ __forceinline__ float head_gate_factor(const float* gate, int ldg, int t, int h) {
+    return gate ? sigmoid_f(gate[(size_t)t * ldg + h]) : 1.0f;
+}
+
+// the column's output row: lane holds dims 16dt + 4g + i; every value is divided by the row's sum, then multiplied by `factor`
 template <int DT>
-__device__ __forceinline__ void store_output(bf16_t* dst, int g, const f32x4_t (&o_tot)[DT], float l_tot) {
+__device__ __forceinline__ void store_output(bf16_t* dst, int g, const f32x4_t (&o_tot)[DT], float l_tot, float factor) {
     const float inv = 1.0f / l_tot;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-        const u32x2_t packed = {(uint32_t)f32_to_bf16(o_tot[dt][0] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][1] * inv) << 16),
-                                (uint32_t)f32_to_bf16(o_tot[dt][2] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][3] * inv) << 16)};
+        const u32x2_t packed = {(uint32_t)f32_to_bf16(o_tot[dt][0] * inv * factor) | ((uint32_t)f32_to_bf16(o_tot[dt][1] * inv * factor) << 16),
+                                (uint32_t)f32_to_bf16(o_tot[dt][2] * inv * factor) | ((uint32_t)f32_to_bf16(o_tot[dt][3] * inv * factor) << 16)};
         *reinterpret_cast<u32x2_t*>(dst + 16 * dt + 4 * g) = packed;
     }
 }
@@ -188,6 +193,8 @@ struct AttnMfmaArgs {
     float* part_ml;         // [slots * 16, 2]: segment max, segment sum
     float scale;
     int n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
+    const float* gate;      // null, or a logit a (row, head): the output is multiplied by its sigmoid
+    int gate_ld;            // the gate rows' stride
 };
 
 // One wave per item, keys and values straight from the pages into the products' operands: the form for decoding rows,
@@ -352,7 +359,7 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
         }
     }
     if constexpr (!PARTIAL) {
-        if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
+        if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot, head_gate_factor(a.gate, a.gate_ld, t, h));
     }
 }
 
@@ -715,7 +722,7 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
         if (more) stage_keys();
         __syncthreads();                       // the next keys are in LDS; nobody reads this segment's values any more
     }
-    if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
+    if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot, head_gate_factor(a.gate, a.gate_ld, t, h));
 }
 
 // Lane l of the wave: 16 bytes from base + offset (bytes, per lane) to LDS at lds + 16 l (lds the same for the whole
@@ -881,7 +888,7 @@ __global__ void __launch_bounds__(64 * AM_TILES128_WAVES) paged_attention_tiles1
         }
         buf ^= 1;
     }
-    if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
+    if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot, head_gate_factor(a.gate, a.gate_ld, t, h));
 }
 
 // The merge's sizes: segments whose weights are formed at a time, segments a round, rounds in flight, and the rows
@@ -1059,7 +1066,8 @@ __device__ __forceinline__ void merge_chunk_weights(const float* base_ml, int c0
 template <int OW, bool SHORT, bool LW>
 __global__ void __launch_bounds__(64 * (OW + (LW ? 1 : 0))) attention_merge_kernel(const int* __restrict__ merges, const int* __restrict__ pos,
                                                                       const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                                      bf16_t* __restrict__ out, int n_heads, int D, int window, int parts) {
+                                                                      bf16_t* __restrict__ out, int n_heads, int D, int window, int parts,
+                                                                      const float* __restrict__ gate, int gate_ld) {
     static_assert(MERGE_CHUNK % (MERGE_DEPTH * MERGE_RING) == 0, "a chunk is a whole number of turns of the ring");
     __shared__ MergeWeights w;
     const int tid = threadIdx.x, wave = tid >> 6;
@@ -1118,7 +1126,7 @@ __global__ void __launch_bounds__(64 * (OW + (LW ? 1 : 0))) attention_merge_kern
         __syncthreads();
         L = w.l_total;
     }
-    if (wave < OW && dim < D) out[((size_t)t * n_heads + h) * D + dim] = f32_to_bf16(O * (1.0f / L));
+    if (wave < OW && dim < D) out[((size_t)t * n_heads + h) * D + dim] = f32_to_bf16(O * (1.0f / L) * head_gate_factor(gate, gate_ld, t, h));
 }
 
 // Rows part_o must have beyond its slots' (see the merge).
@@ -1134,13 +1142,15 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
                                          const int* tables, const int* items, int n_shared, int n_direct, int n_partial, const int* merges,
                                          int n_merges,
                                          void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
-                                         int page_tokens, int max_blocks, int window, int forms, hipStream_t stream) {
+                                         int page_tokens, int max_blocks, int window, int forms, const float* gate, int gate_ld,
+                                         hipStream_t stream) {
     const int wide_items = forms & 1;
+    if (gate && gate_ld < n_heads) return -2;
     if (n_shared + n_direct + n_partial <= 0) return 0;
     if (n_shared % 12) return -2;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
     AttnMfmaArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, (bf16_t*)out, part_o,
-                   part_ml, scale, n_direct, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+                   part_ml, scale, n_direct, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window, gate, gate_ld};
     AttnMfmaArgs sh = a;
     sh.n_items = n_shared;
     a.items = items + (size_t)n_shared * AM_ITEM_INTS;
@@ -1178,7 +1188,7 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
     if (n_merges > 0) {
 #define AM_MERGE(OW, SHORT, LW)                                                                                                \
     hipLaunchKernelGGL((attention_merge_kernel<OW, SHORT, LW>), dim3(n_merges * parts), dim3(64 * (OW + (LW ? 1 : 0))), 0, stream, merges, pos, part_o, part_ml, \
-                       (bf16_t*)out, n_heads, head_dim, window, parts)
+                       (bf16_t*)out, n_heads, head_dim, window, parts, gate, gate_ld)
         if (narrow_merge) {
             const int parts = (head_dim + 63) / 64;
             AM_MERGE(1, false, true);

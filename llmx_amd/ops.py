@@ -74,7 +74,7 @@ def _declare(h) -> None:
         "llmx_attention_partial_pad": [],
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, I, F, P, P, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
-        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P],
+        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P, I, P],
         "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P, I, P],
         "llmx_gate_heads": [P, I, P, I, I, I, I, P],
         "llmx_rmsnorm_add_norm": [P, P, P, F, P, F, P, I, P, I, I, P],
@@ -91,7 +91,7 @@ def _declare(h) -> None:
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
         "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, I, P],
         "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, P],
-        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P],
+        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
@@ -1062,11 +1062,13 @@ def attention_mfma_ok(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bo
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
                     tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0,
-                    plan: Optional[AttentionPlan] = None, scratch=None) -> None:
+                    plan: Optional[AttentionPlan] = None, scratch=None, head_gate: Optional[torch.Tensor] = None) -> None:
     """Causal attention of each row over its request's pages.  With a `plan` (and bfloat16, head_dim a multiple of 16,
     pages of a multiple of 16 tokens, values as wide as keys) the matrix-core kernel runs; `scratch(name, shape, dtype)`
     gives it storage for the partial results of split contexts.  Otherwise the universal kernel runs; it takes values of
-    a width of their own (v_cache [pages, kv_heads, v_dim, page_tokens], out [rows, heads * v_dim])."""
+    a width of their own (v_cache [pages, kv_heads, v_dim, page_tokens], out [rows, heads * v_dim]).  `head_gate`: a float32
+    view [rows, heads] (its rows may be columns of a wider projection): the result of (row, head) is multiplied by the
+    sigmoid of its entry before it is stored, by whichever kernel stores it."""
     rows = q.shape[0]
     n_pages, n_kv_heads, page_tokens, head_dim = k_cache.shape
     v_dim = v_cache.shape[2]
@@ -1077,6 +1079,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         raise KernelError(f"paged_attention: head_dim {head_dim} or value width {v_dim} above {MAX_HEAD_DIM}, or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
     common = (_dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=(n_pages, n_kv_heads, v_dim, page_tokens)),
               _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32))
+    gate_at, gate_ld = _rows_view(head_gate, "head_gate", rows, n_heads) if head_gate is not None else (None, 0)
     if plan is not None and plan.n_items and v_dim == head_dim and attention_mfma_ok(q.dtype, head_dim, page_tokens):
         part_o = part_ml = None
         if plan.n_slots:
@@ -1089,11 +1092,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                                plan.n_items - plan.n_shared - plan.n_direct,
                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
                                                _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), n_heads, n_kv_heads,
-                                               head_dim, page_tokens, tables.shape[1], int(window), (1 if plan.wide_items else 0) | (2 if plan.short_merge else 0), _stream()),
+                                               head_dim, page_tokens, tables.shape[1], int(window), (1 if plan.wide_items else 0) | (2 if plan.short_merge else 0), gate_at, gate_ld,
+                                               _stream()),
                "paged_attention_mfma")
         return
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,
-                                              head_dim, page_tokens, tables.shape[1], int(window), v_dim, _stream()), "paged_attention")
+                                              head_dim, page_tokens, tables.shape[1], int(window), v_dim, gate_at, gate_ld, _stream()), "paged_attention")
 
 
 def _parts_args(z: torch.Tensor, parts: Optional[torch.Tensor]):

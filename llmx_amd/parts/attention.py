@@ -179,9 +179,8 @@ class Attention(Mixer):
         o = step.buf("attention.out", (T, self.o_width), act)
         plan = self._plan(step) if self._mfma(act, cache.k.shape[2]) else None
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
-                            window=int(self.window or 0), plan=plan, scratch=step.buf)
-        if self.head_gate:
-            ops.gate_heads(o, qkv[:, qkv_width:], self.heads)
+                            window=int(self.window or 0), plan=plan, scratch=step.buf,
+                            head_gate=qkv[:, qkv_width:] if self.head_gate else None)      # the gate a head, where the result is stored
         if self.b_o is not None and add_output_bias:
             y = step.buf("attention.projected", (T, self.hidden), torch.float32)
             ops.gemm(o, self.wo, y, scratch=step.buf)

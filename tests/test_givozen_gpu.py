@@ -255,8 +255,7 @@ def _attention_case(dtype, H, G, D, VD, R, scaling, page, length, sharp=None, de
         plan = None
         if VD == D and o.attention_mfma_ok(dtype, D, page):
             plan = o.attention_plan([n], [b], H, G, torch.device("cuda"), 0)
-        o.paged_attention(q, kc, vc, pos, ent, tables, part, scale, H, plan=plan)
-        o.gate_heads(part, rows[:, width:], H)
+        o.paged_attention(q, kc, vc, pos, ent, tables, part, scale, H, plan=plan, head_gate=rows[:, width:])
         out[a:b] = part
     return out.float().cpu(), torch.as_tensor(want)
 
@@ -466,11 +465,12 @@ def test_which_kernels_a_serving_step_takes():
             engine.step([entry])
             for name, count in o.take_launches().items():
                 seen[name] = seen.get(name, 0) + count
-        for name in ("head_norm_rope_kvwrite", "gate_heads", "act.polynorm", "add_rows_vector", "rmsnorm_add", "rmsnorm_add_norm", "rmsnorm",
+        for name in ("head_norm_rope_kvwrite", "act.polynorm", "add_rows_vector", "rmsnorm_add", "rmsnorm_add_norm", "rmsnorm",
                      "moe_combine"):
             assert seen.get(name), f"{dtype}: no launch of {name} ({sorted(seen)})"
-        assert "act.glu" not in seen          # the experts' unit runs in their first product's epilogue
-        assert seen["add_rows_vector"] == 2 * 3 and seen["gate_heads"] == 2 * 8           # three passes, eight layer runs, two steps
+        # the experts' unit runs in their first product's epilogue, the gate a head where the attention stores its result
+        assert "act.glu" not in seen and "gate_heads" not in seen
+        assert seen["add_rows_vector"] == 2 * 3                                          # three passes, two steps
         assert seen["rmsnorm_add_norm"] == 2 * 7 and seen["rmsnorm_add"] == 2 * 8        # seven runs have a feed-forward; its join and the last layer's
         if dtype == "bfloat16":
             assert not any(n.startswith(("gemm_generic", "attention.generic")) for n in seen), sorted(seen)
