@@ -346,6 +346,10 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
     if (norm_w && !llmx_gemm_skinny_f32_normed_ok(M, K)) return -2;
     SkinnyF32Args g{A, W, C, M, N, K, lda, ldc, add, slice_stride, norm_w, norm_eps};
     int chunks = (M + 63) / 64;
+    // a single strip of few slices over many rows (a product of one or a few features): chunks of 64 rows would leave most
+    // of the chip idle, so the rows go in chunks of 16, four times the workgroups (an output's bits depend on K and ks only)
+    const bool thin = N <= 16 && M > 64 && slices * chunks < 128;
+    if (thin) chunks = (M + 15) / 16;
     if (chunks > 1024) chunks = 1024;
     const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks, slices);
     if (M > 64 && N >= 128 && K % 16 == 0 && ks >= 1 && ks <= 16) {
@@ -372,7 +376,7 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
     do {                                                                                                                      \
         if (norm_w)                                                                                                           \
             hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, 1, true>), grid, dim3(64 * KS), (size_t)M * K * sizeof(float), stream, g); \
-        else if (M <= 16) SKF_LAUNCH(KS, 1);                                                                                  \
+        else if (M <= 16 || thin) SKF_LAUNCH(KS, 1);                                                                          \
         else if (M <= 32) SKF_LAUNCH(KS, 2);                                                                                  \
         else SKF_LAUNCH(KS, 4);                                                                                               \
     } while (0)

@@ -193,11 +193,15 @@ extern "C" int llmx_add_rows_vector(float* x, const float* rows, const float* ve
 
 // ---------------------------------------------------------------------------
 // A polynomial of unit-RMS powers between two products: with U(v) = v / sqrt(mean(v^2) + eps) over a row,
-// out = a U(z) + b U(z^2) + c U(z^3) + e, powers element by element, (a, b, c, e) four numbers on the device.  A block a
-// row: the sums of z^2, z^4 and z^6 in one pass (each in the fixed order of strided_squares and block_sum), then the
-// row again (it is still in the caches).  Everything float32; only the result is stored in the activation type.
-#define POLY_THREADS 256
-template <typename TO>
+// out = a U(z) + b U(z^2) + c U(z^3) + e, powers element by element, (a, b, c, e) four numbers on the device.  A block of
+// 1,024 threads a row: the sums of z^2, z^4 and z^6 in one pass (a thread's elements in stride order with fmaf, then
+// block_sum), then the row again.  Rows of at most 16,384 values stay in registers between the two passes, every load asked
+// for before the first sum, so the kernel waits for memory once; longer rows are read again (they are still in the
+// caches).  The same operations in the same order either way.  Everything float32; only the result is stored in the
+// activation type.
+#define POLY_THREADS 1024
+#define POLY_KEPT 16
+template <typename TO, int KEPT>
 __global__ void __launch_bounds__(POLY_THREADS) polynorm_kernel(const float* __restrict__ z, const float* __restrict__ abce, float eps,
                                                               TO* __restrict__ out, int n) {
     __shared__ float scratch[POLY_THREADS / 64];
@@ -205,33 +209,66 @@ __global__ void __launch_bounds__(POLY_THREADS) polynorm_kernel(const float* __r
     const float* row = z + (size_t)r * n;
     const float a = abce[0], b = abce[1], c = abce[2], e = abce[3];
     float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
+    auto add = [&](float v) {
+        const float p2 = v * v, p3 = p2 * v;
+        s2 = fmaf(v, v, s2);
+        s4 = fmaf(p2, p2, s4);
+        s6 = fmaf(p3, p3, s6);
+    };
+    auto factors = [&](float& r1, float& r2, float& r3) {
+        s2 = block_sum<POLY_THREADS / 64>(s2, scratch);
+        s4 = block_sum<POLY_THREADS / 64>(s4, scratch);
+        s6 = block_sum<POLY_THREADS / 64>(s6, scratch);
+        r1 = a / sqrtf(s2 / (float)n + eps);
+        r2 = b / sqrtf(s4 / (float)n + eps);
+        r3 = c / sqrtf(s6 / (float)n + eps);
+    };
+    auto value = [&](float v, float r1, float r2, float r3) {
+        const float p2 = v * v;
+        return ((v * r1 + p2 * r2) + (p2 * v) * r3) + e;
+    };
+    float r1, r2, r3;
+    if (n <= POLY_THREADS * KEPT) {
+        float v[KEPT];
+#pragma unroll
+        for (int u = 0; u < KEPT; ++u) {
+            const int i = threadIdx.x + u * POLY_THREADS;
+            v[u] = i < n ? row[i] : 0.0f;           // an element past the end adds fmaf(0, 0, s) = s
+        }
+#pragma unroll
+        for (int u = 0; u < KEPT; ++u) add(v[u]);
+        factors(r1, r2, r3);
+#pragma unroll
+        for (int u = 0; u < KEPT; ++u) {
+            const int i = threadIdx.x + u * POLY_THREADS;
+            if (i < n) st(out + (size_t)r * n + i, value(v[u], r1, r2, r3));
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < n; i += 4 * POLY_THREADS) {
         float v[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) v[u] = i + u * POLY_THREADS < n ? row[i + u * POLY_THREADS] : 0.0f;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const float p2 = v[u] * v[u], p3 = p2 * v[u];
-            s2 = fmaf(v[u], v[u], s2);
-            s4 = fmaf(p2, p2, s4);
-            s6 = fmaf(p3, p3, s6);
-        }
+        for (int u = 0; u < 4; ++u) add(v[u]);
     }
-    s2 = block_sum<POLY_THREADS / 64>(s2, scratch);
-    s4 = block_sum<POLY_THREADS / 64>(s4, scratch);
-    s6 = block_sum<POLY_THREADS / 64>(s6, scratch);
-    const float r1 = a / sqrtf(s2 / (float)n + eps), r2 = b / sqrtf(s4 / (float)n + eps), r3 = c / sqrtf(s6 / (float)n + eps);
-    for (int i = threadIdx.x; i < n; i += POLY_THREADS) {
-        const float v = row[i], p2 = v * v;
-        st(out + (size_t)r * n + i, ((v * r1 + p2 * r2) + (p2 * v) * r3) + e);
-    }
+    factors(r1, r2, r3);
+    for (int i = threadIdx.x; i < n; i += POLY_THREADS) st(out + (size_t)r * n + i, value(row[i], r1, r2, r3));
 }
 
 extern "C" int llmx_act_polynorm(const float* z, const float* abce, float eps, void* out, int out_dtype, int rows, int n, hipStream_t stream) {
     if (rows <= 0 || n <= 0) return 0;
     llmx_note_launch(LK_ACT_POLYNORM);
-    if (out_dtype == LLMX_F32) hipLaunchKernelGGL(polynorm_kernel<float>, dim3(rows), dim3(POLY_THREADS), 0, stream, z, abce, eps, (float*)out, n);
-    else hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(rows), dim3(POLY_THREADS), 0, stream, z, abce, eps, (bf16_t*)out, n);
+    // half the registers where a row fits them: more rows on a compute unit at a time
+#define POLY_LAUNCH(TO, KEPT) hipLaunchKernelGGL((polynorm_kernel<TO, KEPT>), dim3(rows), dim3(POLY_THREADS), 0, stream, z, abce, eps, (TO*)out, n)
+    if (out_dtype == LLMX_F32) {
+        if (n <= POLY_THREADS * POLY_KEPT / 2) POLY_LAUNCH(float, POLY_KEPT / 2);
+        else POLY_LAUNCH(float, POLY_KEPT);
+    } else {
+        if (n <= POLY_THREADS * POLY_KEPT / 2) POLY_LAUNCH(bf16_t, POLY_KEPT / 2);
+        else POLY_LAUNCH(bf16_t, POLY_KEPT);
+    }
+#undef POLY_LAUNCH
     return LLMX_CHECK_LAUNCH();
 }
 

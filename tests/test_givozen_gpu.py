@@ -51,7 +51,7 @@ def close(got, want, tol, what=""):
 
 # ---------------------------------------------------------------------------
 # kernels alone
-@pytest.mark.parametrize("rows,n", [(1, 8), (5, 21), (3, 1030), (2, 4100)])
+@pytest.mark.parametrize("rows,n", [(1, 8), (5, 21), (3, 1030), (2, 4100), (2, 16384), (2, 16391)])
 def test_polynomial_of_unit_rms_powers(rows, n):
     rng = np.random.default_rng(n)
     o = ops()
