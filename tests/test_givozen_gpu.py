@@ -262,7 +262,7 @@ def _attention_case(dtype, H, G, D, VD, R, scaling, page, length, sharp=None, de
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
 @pytest.mark.parametrize("sizes", [(4, 2, 32, 32, 16, (4.0, 1.0, 4.0, 64), 16), (3, 1, 10, 6, 6, None, 4), (6, 6, 16, 48, 16, (8.0, 2.0, 16.0, 32), 16),
-                                   (8, 2, 64, 64, 16, (8.0, 1.0, 4.0, 128), 16), (1, 1, 128, 128, 0, None, 16), (2, 1, 48, 16, 48, None, 8)])
+                                   (8, 4, 64, 64, 32, (4.0, 1.0, 8.0, 128), 16), (1, 1, 128, 128, 0, None, 16), (2, 1, 48, 16, 48, None, 8)])
 def test_attention_with_biases_temperature_and_gate_over_shuffled_pages(dtype, sizes):
     H, G, D, VD, R, scaling, page = sizes
     scale = 0.5 / D ** 0.5          # scores of the same moderate spread whatever the head's width (the sharp cases are below)
