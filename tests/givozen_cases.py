@@ -78,9 +78,35 @@ CONFIG_D = {
     ],
     "loop": {"start": 1, "stop": 2, "times": 1},
 }
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
-PAGES = {"A": 16, "B": 4, "C": 16, "D": 16}
-SEEDS = {"A": 21, "B": 22, "C": 23, "D": 24}
+# E: the repeated run reaches the model's end and holds a layer without feed-forward; one pick of sixteen experts beside a
+#    shared expert wider than they are; grouped heads with values twice as wide as keys beside a mixer with one key head.
+_E_WIDE = _mixer(6, 3, 32, 64, 0.21, 20000.0, 32, (4.0, 1.0, 8.0, 256))
+_E_ONE = _mixer(4, 1, 48, 48, 0.17, 3000.0, 24)
+CONFIG_E = {
+    "architecture": "Givozen", "vocab": 700, "width": 192, "norm": {"eps": 1e-5},
+    "layers": [
+        _layer(_E_WIDE, _moe(4, 2, 80, 1.2)),
+        _layer(_E_ONE, {"kind": "dense", "ff": 320}),
+        _layer(_E_WIDE, None),
+        _layer(_E_ONE, _moe(16, 1, 48, 4.0, (112, 0.9))),
+    ],
+    "loop": {"start": 2, "stop": 4, "times": 3},
+}
+# F: heads of 128 and of 64 (the matrix-core attention's widest kernels, prompt tiles and split contexts), the first layer
+#    alone repeated, every one of six experts picked in the last layer.
+_F_WIDE = _mixer(4, 2, 128, 128, 0.088, 500000.0, 64, (8.0, 1.0, 4.0, 512))
+CONFIG_F = {
+    "architecture": "Givozen", "vocab": 512, "width": 384, "norm": {"eps": 1e-6},
+    "layers": [
+        _layer(_F_WIDE, _moe(6, 2, 96, 3.0, (160, 1.5))),
+        _layer(_mixer(6, 3, 64, 64, 0.125, 10000.0, 32, (2.0, 1.0, 2.0, 128)), {"kind": "dense", "ff": 640}),
+        _layer(_F_WIDE, _moe(6, 6, 96, 2.0)),
+    ],
+    "loop": {"start": 0, "stop": 1, "times": 2},
+}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D, "E": CONFIG_E, "F": CONFIG_F}
+PAGES = {"A": 16, "B": 4, "C": 16, "D": 16, "E": 16, "F": 16}
+SEEDS = {"A": 21, "B": 22, "C": 23, "D": 24, "E": 25, "F": 26}
 
 
 def write_folder(config: dict, seed: int, folder: str, edit=None) -> str:
