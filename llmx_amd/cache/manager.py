@@ -26,6 +26,22 @@ class GroupSpec:
     page_tokens: int
     n_pages: int
     window: Optional[int] = None  # None: every key is kept; w: a row at p reads keys p-w+1 .. p
+    keep_first: int = 0           # under a window: positions 0 .. keep_first-1 stay readable too (their pages are kept)
+    chunk: Optional[int] = None   # c: a row at p reads keys floor(p / c) * c .. p only
+
+    @property
+    def releases(self) -> bool:
+        """Whether committed steps give back pages that no later row can read."""
+        return self.window is not None or self.chunk is not None
+
+    def first_read(self, position: int) -> int:
+        """The lowest position, beyond the kept first ones, that a row at `position` or later can read."""
+        lo = 0
+        if self.window is not None:
+            lo = max(lo, position - self.window + 1)
+        if self.chunk is not None:
+            lo = max(lo, (position // self.chunk) * self.chunk)
+        return lo
 
     def pages_for(self, tokens: int) -> int:
         return -(-tokens // self.page_tokens)
@@ -33,15 +49,17 @@ class GroupSpec:
     def peak_pages(self, total_tokens: int, step_tokens: int) -> int:
         """Most pages a request of `total_tokens` holds at once when a step brings at most `step_tokens` of its tokens."""
         whole = self.pages_for(total_tokens)
-        if self.window is None:
+        if not self.releases:
             return whole
-        return min(whole, self.pages_for(self.window + step_tokens) + 1)
+        span = min(self.window if self.window is not None else self.chunk, self.chunk if self.chunk is not None else self.window)
+        kept = self.pages_for(self.keep_first) if self.keep_first else 0
+        return min(whole, self.pages_for(span + step_tokens) + 1 + kept)
 
     def pool_pages(self, total_tokens: int, requests: int, step_tokens: Optional[int]) -> int:
         """Pages of a pool made for `total_tokens` tokens: all of them for a group that keeps every key; for a window,
         when the most tokens a step brings of one request is known, what `requests` requests can hold at once."""
         whole = self.pages_for(total_tokens)
-        if self.window is None or step_tokens is None:
+        if not self.releases or step_tokens is None:
             return whole
         return min(whole, requests * self.peak_pages(total_tokens, step_tokens))
 
@@ -134,13 +152,15 @@ class CacheManager:
             r.slot, r.shadow = r.shadow, -1
         for gi, g in enumerate(self.groups):
             r.taken[gi].clear()
-            if g.window is not None:
-                # the next row sits at position >= length and reads keys >= length - window + 1
-                dead_below = r.length - g.window + 1
+            if g.releases:
+                # the next row sits at position >= length and reads keys >= first_read(length), and the kept first ones
+                dead_below = g.first_read(r.length)
                 table = r.tables[gi]
                 for i in range(len(table)):
                     if (i + 1) * g.page_tokens > dead_below:
                         break
+                    if i * g.page_tokens < g.keep_first:
+                        continue
                     if table[i] >= 0:
                         self.pools[gi].release(table[i])
                         table[i] = -1
@@ -163,14 +183,14 @@ class CacheManager:
         if not 0 <= length <= r.length:
             raise CacheLogicError(f"cache: request {request!r} holds {r.length} tokens and cannot be taken back to {length}")
         for gi, g in enumerate(self.groups):
-            if g.window is None:
+            if not g.releases:
                 continue
             table = r.tables[gi]
-            first = max(0, length - g.window + 1)     # the row at `length` reads keys first .. length - 1
+            first = g.first_read(length)     # the row at `length` reads keys first .. length - 1
             for i in range(first // g.page_tokens, g.pages_for(length)):
                 if table[i] < 0:
                     raise CacheLogicError(f"cache: request {request!r} cannot be taken back to {length} tokens: {g.name} keeps the last "
-                                          f"{g.window} keys only and has given back the page of position {i * g.page_tokens}")
+                                          f"{g.window if g.window is not None else g.chunk} keys only and has given back the page of position {i * g.page_tokens}")
         for gi, g in enumerate(self.groups):
             table = r.tables[gi]
             keep = g.pages_for(length)

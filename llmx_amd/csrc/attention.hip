@@ -254,13 +254,18 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
 }
 
 // ---------------------------------------------------------------------------
-// The same step for heads that are normed one by one: one wave a (row, head).  The projections' biases (optional) are added
+// The same step for heads that are treated one by one: one wave a (row, head).  The projections' biases (optional) are added
 // first; each q and k head is then RMS-normed over its head_dim values with a weight of head_dim values shared by all
 // heads (norm_mode QKNORM_HEAD; QKNORM_NONE: no norm), its first rotary_dim dims are rotated, and k and v go to the row's
-// page.  Values have a width of their own (v_dim) and are not normed or rotated.  The row is q (H*D) | k (G*D) | v (G*VD).
+// page.  Values have a width of their own (v_dim) and are not rotated.  The row is q (HQ*D) | k (HK*D) | v (HV*VD).
+// There may be more key heads than value heads (HK a multiple of HV: several score maps over one set of values, key head
+// kk going with value head kk / (HK / HV)); the first key head of a value head writes the value.
+// v_source 1: the row has no v columns; a value head is its key head as projected (with its bias, before norm and
+// rotation), so VD = D and HK = HV.  v_norm 1: a value head is divided by its root mean square over VD (eps inside the
+// root, no weight) before it is stored.
 struct HeadPrepArgs {
     const float* qkv;
-    const float* bias;       // [H*D + G*D + G*VD] or null
+    const float* bias;       // [HQ*D + HK*D + HV*VD] or null
     const float* q_weight;   // [D]
     const float* k_weight;   // [D]
     const float* cos_sin;
@@ -268,37 +273,40 @@ struct HeadPrepArgs {
     const int* row_entry;
     const int* tables;
     void* q_out;
-    void* k_cache;           // [page][kv_head][token][D]
-    void* v_cache;           // [page][kv_head][VD][token]
+    void* k_cache;           // [page][key head][token][D]
+    void* v_cache;           // [page][value head][VD][token]
     float eps;
-    int n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode;
+    int n_heads, n_k_heads, n_v_heads, head_dim, v_dim, rotary_dim, norm_mode;
     int page_tokens, max_blocks, write_kv, pairing;
-    const float* q_scale;    // [H] or null: a factor a query head on the rotated q (a temperature a head on its scores)
+    const float* q_scale;    // [HQ] or null: a factor a query head on the rotated q (a temperature a head on its scores)
     int ld;                  // row stride of qkv (at least its width: further columns of the projection may follow v)
+    int v_source, v_norm;
 };
 
 template <typename T>
 __global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs a) {
     __shared__ float head[ATT_PREP_MAX_D];
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
-    const int D = a.head_dim, VD = a.v_dim, H = a.n_heads, G = a.n_kv_heads;
-    const int width = H * D + G * D + G * VD;
+    const int D = a.head_dim, VD = a.v_dim, H = a.n_heads, G = a.n_k_heads, GV = a.n_v_heads;
+    const int width = H * D + G * D + (a.v_source ? 0 : GV * VD);
     const bool is_q = hh < H;
     if (!is_q && !a.write_kv) return;
     const int g = hh - H;
     const int col0 = is_q ? hh * D : H * D + g * D;
     const float* row = a.qkv + (size_t)t * (a.ld > width ? a.ld : width);
     const int p = a.pos[t];
-    float x[ATT_PREP_MAX_D / 64];
+    float x[ATT_PREP_MAX_D / 64], raw[ATT_PREP_MAX_D / 64];
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
         x[i] = d < D ? row[col0 + d] + (a.bias ? a.bias[col0 + d] : 0.0f) : 0.0f;
+        raw[i] = x[i];
         ss = fmaf(x[i], x[i], ss);
     }
+    const float sum_sq = wave_sum(ss);
     if (a.norm_mode == QKNORM_HEAD) {
-        const float r = 1.0f / sqrtf(wave_sum(ss) / (float)D + a.eps);
+        const float r = 1.0f / sqrtf(sum_sq / (float)D + a.eps);
         const float* w = is_q ? a.q_weight : a.k_weight;
 #pragma unroll
         for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
@@ -334,27 +342,53 @@ __global__ void __launch_bounds__(64) head_norm_rope_kvwrite_kernel(HeadPrepArgs
         if (is_q) st((T*)a.q_out + (size_t)t * H * D + col0 + d, a.q_scale ? y * q_factor : y);
         else st((T*)a.k_cache + (head_at * a.page_tokens + slot) * D + d, y);
     }
-    if (!is_q) {
-        const int vcol = H * D + G * D + g * VD;
-        for (int d = lane; d < VD; d += 64)
-            st((T*)a.v_cache + (head_at * VD + d) * a.page_tokens + slot, row[vcol + d] + (a.bias ? a.bias[vcol + d] : 0.0f));
+    const int share = G / GV;     // key heads that go with one value head
+    if (!is_q && g % share == 0) {
+        const int gv = g / share;
+        const size_t v_at = (size_t)page * GV + gv;
+        if (a.v_source) {          // the value is the key as projected: VD = D
+            const float r = a.v_norm ? 1.0f / sqrtf(sum_sq / (float)D + a.eps) : 1.0f;
+#pragma unroll
+            for (int i = 0; i < ATT_PREP_MAX_D / 64; ++i) {
+                const int d = lane + 64 * i;
+                if (d < D) st((T*)a.v_cache + (v_at * VD + d) * a.page_tokens + slot, a.v_norm ? raw[i] * r : raw[i]);
+            }
+        } else {
+            const int vcol = H * D + G * D + gv * VD;
+            float r = 1.0f;
+            if (a.v_norm) {
+                float vs = 0.0f;
+                for (int d = lane; d < VD; d += 64) {
+                    const float v = row[vcol + d] + (a.bias ? a.bias[vcol + d] : 0.0f);
+                    vs = fmaf(v, v, vs);
+                }
+                r = 1.0f / sqrtf(wave_sum(vs) / (float)VD + a.eps);
+            }
+            for (int d = lane; d < VD; d += 64) {
+                const float v = row[vcol + d] + (a.bias ? a.bias[vcol + d] : 0.0f);
+                st((T*)a.v_cache + (v_at * VD + d) * a.page_tokens + slot, a.v_norm ? v * r : v);
+            }
+        }
     }
 }
 
 extern "C" int llmx_head_norm_rope_kvwrite(const float* qkv, const float* bias, const float* q_weight, const float* k_weight, const float* cos_sin,
                                            const int* pos, const int* row_entry, const int* tables, void* q_out, void* k_cache, void* v_cache,
-                                           int dtype, float eps, int rows, int n_heads, int n_kv_heads, int head_dim, int v_dim, int rotary_dim,
+                                           int dtype, float eps, int rows, int n_heads, int n_k_heads, int head_dim, int v_dim, int rotary_dim,
                                            int norm_mode, int page_tokens, int max_blocks, int write_kv, int pairing, const float* q_scale,
-                                           int ld, hipStream_t stream) {
+                                           int ld, int n_v_heads, int v_source, int v_norm, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_HEAD) return -2;
     if (pairing != ROPE_HALVES && pairing != ROPE_INTERLEAVED) return -2;
     if (head_dim < 1 || head_dim > ATT_PREP_MAX_D || v_dim < 1 || rotary_dim > head_dim || rotary_dim % 2) return -2;
     if (norm_mode == QKNORM_HEAD && (!q_weight || !k_weight)) return -2;
+    if (n_v_heads < 1 || n_k_heads % n_v_heads) return -2;
+    if (v_source && (v_dim != head_dim || n_k_heads != n_v_heads)) return -2;
     HeadPrepArgs a{qkv, bias, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
-                   n_heads, n_kv_heads, head_dim, v_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, pairing, q_scale, ld};
+                   n_heads, n_k_heads, n_v_heads, head_dim, v_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, pairing, q_scale, ld,
+                   v_source, v_norm};
     llmx_note_launch(LK_HEAD_NORM_ROPE_KVWRITE);
-    const dim3 grid(rows, n_heads + n_kv_heads);
+    const dim3 grid(rows, n_heads + n_k_heads);
     if (dtype == LLMX_F32) hipLaunchKernelGGL(head_norm_rope_kvwrite_kernel<float>, grid, dim3(64), 0, stream, a);
     else hipLaunchKernelGGL(head_norm_rope_kvwrite_kernel<bf16_t>, grid, dim3(64), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
@@ -384,109 +418,148 @@ extern "C" int llmx_gate_heads(void* o, int dtype, const float* gate, int ldg, i
 }
 
 // ---------------------------------------------------------------------------
-// Universal paged attention: one wave per (row, head).  Keys lo..p of the row's request are walked in tiles of 64 in
-// position order with an online softmax; lo = max(0, p - window + 1) under a window, else 0.  Lane j of a tile owns key
-// lo + 64*tile + j for the scores; for the value sum lane d owns dims d, d+64, ... and walks the tile's keys in order.
+// Universal paged attention: one wave per (row, head, map).  The keys a row at position p sees are walked in tiles of 64 in
+// position order with an online softmax.  What it sees: keys lo..p, with lo = max(0, p - window + 1) under a window,
+// lo = floor(p / chunk) * chunk under chunks (counted from position 0 of the request), else 0; and, before those, the keys
+// 0..min(keep_first, lo) - 1 (a window that also keeps a request's first tokens, at their true positions).  Lane j of a tile
+// owns one key for the scores; for the value sum lane d owns dims d, d+64, ... and walks the tile's keys in order.
+// A score is q.k * scale, then softcap * tanh(score / softcap) (softcap > 0), then minus slopes[h] * (p - j) (slopes given).
+// `sink` (a logit a head) enters the softmax's denominator only.  `maps` > 1: a head has several score maps over one set of
+// values: q holds [head][map][D], the key cache [kv head][map] heads, and the output [head][map][VD].
 // A row's arithmetic depends on its own position and request only.  Values may have a width of their own (v_dim).
 struct AttnArgs {
-    const void* q;  // [T, n_heads, head_dim]
+    const void* q;  // [T, n_heads * maps, head_dim]
     const void* k_cache;
     const void* v_cache;
     const int* pos;
     const int* row_entry;
     const int* tables;
-    void* out;  // [T, n_heads * head_dim]
+    void* out;  // [T, n_heads * maps * v_dim]
     float scale;
     int n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
     int v_dim;   // width of a value head (the output's too); keys and queries have head_dim
-    const float* gate;  // null, or a float32 logit a (row, head), row stride gate_ld: the output is multiplied by its sigmoid
+    const float* gate;  // null, or float32 logits, row stride gate_ld: the output is multiplied by their sigmoid
     int gate_ld;
+    int gate_wide;       // 0: a logit a (row, head); 1: a logit a (row, head, value dim)
+    int keep_first, chunk, maps;
+    float softcap;
+    const float* slopes;   // [n_heads] or null
+    const float* sink;     // [n_heads] or null
 };
 
 #define ATT_MAX_D 256
 
-template <typename T>
+template <typename T, typename TO>
 __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a) {
     __shared__ float qs[ATT_MAX_D];
     __shared__ float ps[64];
-    __shared__ int heads_at[64];  // page * kv_heads + kv_head of each key of the tile
+    __shared__ int heads_at[64];  // page * value heads + value head of each key of the tile
     __shared__ int slots[64];     // its place in the page
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int D = a.head_dim, VD = a.v_dim;
+    const int t = blockIdx.x, hm = blockIdx.y, lane = threadIdx.x;
+    const int D = a.head_dim, VD = a.v_dim, M = a.maps;
+    const int h = hm / M, map = hm - h * M;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
+    const int key_heads = a.n_kv_heads * M, key_head = kvh * M + map;
     const int p = a.pos[t];
     const int* table = a.tables + (size_t)a.row_entry[t] * a.max_blocks;
-    const T* q = (const T*)a.q + ((size_t)t * a.n_heads + h) * D;
+    const T* q = (const T*)a.q + ((size_t)t * a.n_heads * M + hm) * D;
     const T* kc = (const T*)a.k_cache;
     const T* vc = (const T*)a.v_cache;
     for (int d = lane; d < D; d += 64) qs[d] = ld(q + d);
     __syncthreads();
 
-    const int lo = (a.window > 0 && p - a.window + 1 > 0) ? p - a.window + 1 : 0;
+    int lo = 0;
+    if (a.window > 0 && p - a.window + 1 > 0) lo = p - a.window + 1;
+    if (a.chunk > 0) lo = max(lo, (p / a.chunk) * a.chunk);
+    const int kept = min(a.keep_first, lo);
+    const float slope = a.slopes ? a.slopes[h] : 0.0f;
     float m = -INFINITY, l = 0.0f;
     float acc[ATT_MAX_D / 64];
 #pragma unroll
     for (int i = 0; i < ATT_MAX_D / 64; ++i) acc[i] = 0.0f;
 
-    for (int j0 = lo; j0 <= p; j0 += 64) {
-        const int j = j0 + lane;
-        float s = -INFINITY;
-        int head_at = 0, slot = 0;
-        if (j <= p) {
-            const int page = table[j / a.page_tokens];
-            head_at = page * a.n_kv_heads + kvh;
-            slot = j % a.page_tokens;
-            const size_t base = ((size_t)head_at * a.page_tokens + slot) * D;
-            float dot = 0.0f;
-            for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld(kc + base + d), dot);
-            s = dot * a.scale;
-        }
-        const float tile_max = wave_max(s);
-        const float m_new = fmaxf(m, tile_max);
-        const float w = j <= p ? expf(s - m_new) : 0.0f;
-        const float correction = expf(m - m_new);  // 0 on the first tile (m = -inf)
-        // the tile's weights summed in key order by every lane alike
-        ps[lane] = w;
-        heads_at[lane] = head_at;
-        slots[lane] = slot;
-        __syncthreads();
-        float tile_sum = 0.0f;
-        const int n = min(64, p - j0 + 1);
-        for (int i = 0; i < n; ++i) tile_sum += ps[i];
-        l = l * correction + tile_sum;
-#pragma unroll
-        for (int i = 0; i < ATT_MAX_D / 64; ++i) {
-            const int d = lane + 64 * i;
-            if (d < VD) {
-                float v = acc[i] * correction;
-                for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + ((size_t)heads_at[jj] * VD + d) * a.page_tokens + slots[jj]), v);
-                acc[i] = v;
+    for (int range = kept > 0 ? 0 : 1; range < 2; ++range) {
+        const int begin = range == 0 ? 0 : lo, end = range == 0 ? kept : p + 1;   // keys begin .. end - 1
+        for (int j0 = begin; j0 < end; j0 += 64) {
+            const int j = j0 + lane;
+            float s = -INFINITY;
+            int head_at = 0, slot = 0;
+            if (j < end) {
+                const int page = table[j / a.page_tokens];
+                slot = j % a.page_tokens;
+                head_at = page * a.n_kv_heads + kvh;
+                const size_t base = (((size_t)page * key_heads + key_head) * a.page_tokens + slot) * D;
+                float dot = 0.0f;
+                for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld(kc + base + d), dot);
+                s = dot * a.scale;
+                if (a.softcap > 0.0f) s = a.softcap * tanhf(s / a.softcap);
+                if (a.slopes) s = s - slope * (float)(p - j);
             }
+            const float tile_max = wave_max(s);
+            const float m_new = fmaxf(m, tile_max);
+            const float w = j < end ? expf(s - m_new) : 0.0f;
+            const float correction = expf(m - m_new);  // 0 on the first tile (m = -inf)
+            // the tile's weights summed in key order by every lane alike
+            ps[lane] = w;
+            heads_at[lane] = head_at;
+            slots[lane] = slot;
+            __syncthreads();
+            float tile_sum = 0.0f;
+            const int n = min(64, end - j0);
+            for (int i = 0; i < n; ++i) tile_sum += ps[i];
+            l = l * correction + tile_sum;
+#pragma unroll
+            for (int i = 0; i < ATT_MAX_D / 64; ++i) {
+                const int d = lane + 64 * i;
+                if (d < VD) {
+                    float v = acc[i] * correction;
+                    for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + ((size_t)heads_at[jj] * VD + d) * a.page_tokens + slots[jj]), v);
+                    acc[i] = v;
+                }
+            }
+            m = m_new;
+            __syncthreads();
         }
-        m = m_new;
-        __syncthreads();
     }
-    T* out = (T*)a.out + ((size_t)t * a.n_heads + h) * VD;
-    const float factor = a.gate ? sigmoid_f(a.gate[(size_t)t * a.gate_ld + h]) : 1.0f;
+    float shrink = 1.0f;
+    if (a.sink) {       // one more logit in the denominator: no key, no value
+        const float sk = a.sink[h];
+        const float top = fmaxf(m, sk);
+        shrink = expf(m - top);
+        l = l * shrink + expf(sk - top);
+    }
+    TO* out = (TO*)a.out + ((size_t)t * a.n_heads * M + hm) * VD;
+    const float head_factor = (a.gate && !a.gate_wide) ? sigmoid_f(a.gate[(size_t)t * a.gate_ld + h]) : 1.0f;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
-        if (d < VD) st(out + d, acc[i] / l * factor);
+        if (d < VD) {
+            float y = a.sink ? acc[i] * shrink / l : acc[i] / l;
+            if (a.gate) y = y * (a.gate_wide ? sigmoid_f(a.gate[(size_t)t * a.gate_ld + (size_t)h * VD + d]) : head_factor);
+            st(out + d, y);
+        }
     }
 }
 
+// `out_dtype`: the output's type where it differs from the cache's (several maps are joined in float32 by a later kernel).
 extern "C" int llmx_paged_attention_generic(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
                                             const int* tables, void* out, int dtype, float scale, int rows, int n_heads, int n_kv_heads,
                                             int head_dim, int page_tokens, int max_blocks, int window, int v_dim, const float* gate, int gate_ld,
-                                            hipStream_t stream) {
+                                            int gate_wide, int keep_first, int chunk, int maps, float softcap, const float* slopes,
+                                            const float* sink, int out_dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (head_dim > ATT_MAX_D || v_dim > ATT_MAX_D || v_dim < 1 || n_heads % n_kv_heads || (gate && gate_ld < n_heads)) return -2;
+    if (head_dim > ATT_MAX_D || v_dim > ATT_MAX_D || v_dim < 1 || n_heads % n_kv_heads) return -2;
+    if (gate && gate_ld < (gate_wide ? n_heads * v_dim : n_heads)) return -2;
+    if (maps < 1 || keep_first < 0 || chunk < 0 || window < 0 || (maps > 1 && gate) || (keep_first > 0 && chunk > 0)) return -2;
     AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window, v_dim,
-               gate, gate_ld};
+               gate, gate_ld, gate_wide, keep_first, chunk, maps, softcap, slopes, sink};
     llmx_note_launch(LK_ATTENTION_GENERIC);
+    const dim3 grid(rows, n_heads * maps);
     if (dtype == LLMX_F32)
-        hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(rows, n_heads), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL((paged_attention_generic_kernel<float, float>), grid, dim3(64), 0, stream, a);
+    else if (out_dtype == LLMX_F32)
+        hipLaunchKernelGGL((paged_attention_generic_kernel<bf16_t, float>), grid, dim3(64), 0, stream, a);
     else
-        hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, dim3(rows, n_heads), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL((paged_attention_generic_kernel<bf16_t, bf16_t>), grid, dim3(64), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
 }

@@ -240,13 +240,15 @@ __device__ __forceinline__ void rms_rows_as_1024(const float* __restrict__ X, si
 // xIELU with two learned numbers (p, q) read from the device: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q))
 // (e^z - 1 - z) + z/2.  Both go through these two functions, so a product with the activation gives the bits of the product
 // followed by the activation's kernel.
-enum : int { LLMX_ACT_NONE = 0, LLMX_ACT_XIELU = 1 };
+// RELU2: max(z, 0)^2, no numbers.
+enum : int { LLMX_ACT_NONE = 0, LLMX_ACT_XIELU = 1, LLMX_ACT_RELU2 = 2 };
+__host__ __device__ __forceinline__ bool llmx_act_reads_params(int kind) { return kind == LLMX_ACT_XIELU; }
 __device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.0f); }
 // The activation's numbers as a kernel reads them at its start (uniform loads, long before the epilogue needs them).
 struct ActParams {
     float p, q;
     __device__ __forceinline__ ActParams(int kind, const float* __restrict__ params) : p(0.0f), q(0.0f) {
-        if (kind != LLMX_ACT_NONE) {
+        if (llmx_act_reads_params(kind)) {
             p = params[0];
             q = params[1];
         }
@@ -264,13 +266,19 @@ struct ActFn {
     __device__ __forceinline__ ActFn(int kind_, const float* __restrict__ params) : ActFn(kind_, ActParams(kind_, params)) {}
     __device__ __forceinline__ float operator()(float v) const {
         if (kind == LLMX_ACT_XIELU) return v > 0.0f ? a * v * v + 0.5f * v : b * (expm1f(v) - v) + 0.5f * v;
+        if (kind == LLMX_ACT_RELU2) {
+            const float r = fmaxf(v, 0.0f);
+            return r * r;
+        }
         return v;
     }
 };
 
 // A gated unit of two pre-activations (gate, up), as the products' gated epilogue and the kernel of its own compute it.
 // SILU: silu(gate) * up.  CLAMPED: g = min(gate, limit), u = clamp(up, -limit, limit); g sigmoid(1.702 g) (u + 1).
-enum : int { LLMX_GLU_SILU = 0, LLMX_GLU_CLAMPED = 1 };
+// GELU_TANH: g/2 (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * up.
+enum : int { LLMX_GLU_SILU = 0, LLMX_GLU_CLAMPED = 1, LLMX_GLU_GELU_TANH = 2 };
+__device__ __forceinline__ float gelu_tanh_f(float g) { return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))); }
 __device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
 struct GluFn {
     int kind;
@@ -281,6 +289,7 @@ struct GluFn {
             const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
             return (g / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
         }
+        if (kind == LLMX_GLU_GELU_TANH) return gelu_tanh_f(gate) * up;
         return (gate / (1.0f + expf(-gate))) * up;
     }
 };

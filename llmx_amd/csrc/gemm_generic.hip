@@ -174,7 +174,7 @@ extern "C" int llmx_gemm_generic(const void* A, int a_dtype, const void* W, int 
                epi == EPI_STORE ? act : LLMX_ACT_NONE, act_params,
                GluArgs{epi == EPI_SWIGLU ? glu_kind : LLMX_GLU_SILU, glu_limit, epi == EPI_SWIGLU ? glu_row_scale : nullptr,
                        epi == EPI_SWIGLU ? glu_row_gate : nullptr, glu_row_gate_ld}};
-    if (act != LLMX_ACT_NONE && (epi != EPI_STORE || !act_params)) return -2;
+    if (act != LLMX_ACT_NONE && (epi != EPI_STORE || (llmx_act_reads_params(act) && !act_params))) return -2;
     dim3 grid;
     grid.x = (N + GT_BN - 1) / GT_BN;
     if (n_groups) {

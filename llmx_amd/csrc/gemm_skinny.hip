@@ -424,7 +424,7 @@ extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dty
                  w_group_stride, up_offset, X, norm_w, norm_eps, x_rows, epi == SK_STORE ? act : LLMX_ACT_NONE, act_params,
                  GluArgs{epi == SK_SWIGLU ? glu_kind : LLMX_GLU_SILU, glu_limit, epi == SK_SWIGLU ? glu_row_scale : nullptr,
                          epi == SK_SWIGLU ? glu_row_gate : nullptr, glu_row_gate_ld}};
-    if (act != LLMX_ACT_NONE && (epi != SK_STORE || !act_params)) return -2;
+    if (act != LLMX_ACT_NONE && (epi != SK_STORE || (llmx_act_reads_params(act) && !act_params))) return -2;
     dim3 grid((N + 15) / 16, grouped ? max_active : 1, 1);
     int mt = 1;
     if (!grouped && epi != SK_SWIGLU) mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);

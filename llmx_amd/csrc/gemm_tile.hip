@@ -853,7 +853,7 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
                w_group_stride, up_offset, 0, ks, 64, nullptr, 0, 0, epi == TL_STORE ? act : LLMX_ACT_NONE, act_params,
                GluArgs{epi == TL_SWIGLU ? glu_kind : LLMX_GLU_SILU, glu_limit, epi == TL_SWIGLU ? glu_row_scale : nullptr,
                        epi == TL_SWIGLU ? glu_row_gate : nullptr, glu_row_gate_ld}};
-    if (act != LLMX_ACT_NONE && (epi != TL_STORE || !act_params)) return -2;
+    if (act != LLMX_ACT_NONE && (epi != TL_STORE || (llmx_act_reads_params(act) && !act_params))) return -2;
     auto launch = [&](int form, int tiles_y) -> int {
         g.bm = form_rows(form);
         g.m_tiles = (M + g.bm - 1) / g.bm;

@@ -353,36 +353,165 @@ extern "C" int llmx_state_scan(const float* q, int ldq, const float* k, int ldk,
 }
 
 // ---------------------------------------------------------------------------
-// The read-out's gated norm, one wave a (row, head): out = o / sqrt(mean(o^2) + eps) * w * gate(z), gate = sigmoid or silu
-// of the gate's pre-activation z (a float32 view with its own row stride); out in the activation type for the output
-// projection.
+// The read-out's gated norm, one wave a (row, head): out = x / sqrt(mean(x^2) + eps) * w * gate(z) * post, gate = sigmoid or
+// silu of the gate's pre-activation z (a float32 view with its own row stride; null: no gate); out in the activation type
+// for the output projection.  The head's values x come from o, whose heads start `o_head` floats apart:
+//   x_j = o_j                                               plainly;
+//   x_j = o_j - lambda * o_(sub + j)                        sub > 0: a second map of the head, `sub` floats on, taken off;
+//   x_j = o_j / (max(|o_V|, den_floor[t, h]) + 1e-6)        den_floor given: the head's V values are followed by their
+//                                                           denominator, which is kept away from zero.
+// w: null (no weight), [V] shared by the heads, or (w_wide) [H * V].
 enum : int { GATE_SIGMOID = 0, GATE_SILU = 1 };
 
+struct HeadNormArgs {
+    const float* o;
+    int o_head;
+    const float* w;
+    int w_wide;
+    const float* z;
+    int ldz;
+    float eps;
+    int H, V, gate, sub;
+    float lambda, post;
+    const float* den_floor;
+};
+
 template <typename TO>
-__global__ void __launch_bounds__(64) head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, const float* __restrict__ z,
-                                                          int ldz, TO* __restrict__ out, float eps, int H, int V, int gate) {
+__global__ void __launch_bounds__(64) head_norm_gate_kernel(HeadNormArgs a, TO* __restrict__ out) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const float* row = o + ((size_t)t * H + h) * V;
+    const int H = a.H, V = a.V;
+    const float* row = a.o + ((size_t)t * H + h) * a.o_head;
+    float den = 1.0f;
+    if (a.den_floor) den = fmaxf(fabsf(row[V]), a.den_floor[(size_t)t * H + h]) + 1e-6f;
+    auto value = [&](int j) {
+        float x = row[j];
+        if (a.sub > 0) x = x - a.lambda * row[a.sub + j];
+        if (a.den_floor) x = x / den;
+        return x;
+    };
     float ss = 0.0f;
-    for (int j = lane; j < V; j += 64) ss = fmaf(row[j], row[j], ss);
-    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
-    const float* zr = z + (size_t)t * ldz + (size_t)h * V;
+    for (int j = lane; j < V; j += 64) {
+        const float x = value(j);
+        ss = fmaf(x, x, ss);
+    }
+    const float r = 1.0f / sqrtf(wave_sum(ss) / (float)V + a.eps);
+    const float* zr = a.z ? a.z + (size_t)t * a.ldz + (size_t)h * V : nullptr;
+    const float* w = a.w ? (a.w_wide ? a.w + (size_t)h * V : a.w) : nullptr;
     TO* dst = out + ((size_t)t * H + h) * V;
     for (int j = lane; j < V; j += 64) {
-        const float x = zr[j];
-        const float g = gate == GATE_SIGMOID ? sigmoid_ls(x) : x * sigmoid_ls(x);
-        st(dst + j, row[j] * r * w[j] * g);
+        float y = value(j) * r;
+        if (w) y = y * w[j];
+        if (zr) {
+            const float x = zr[j];
+            y = y * (a.gate == GATE_SIGMOID ? sigmoid_ls(x) : x * sigmoid_ls(x));
+        }
+        if (a.post != 1.0f) y = y * a.post;
+        st(dst + j, y);
     }
 }
 
 extern "C" int llmx_head_norm_gate(const float* o, const float* w, const float* z, int ldz, void* out, int out_dtype, float eps, int rows, int H,
-                                   int V, int gate, hipStream_t stream) {
+                                   int V, int gate, int o_head, int w_wide, int sub, float lambda, float post, const float* den_floor,
+                                   hipStream_t stream) {
     if (rows <= 0) return 0;
     if (H < 1 || V < 1 || (gate != GATE_SIGMOID && gate != GATE_SILU)) return -2;
+    if (o_head < V || sub < 0 || (sub > 0 && (den_floor || o_head < sub + V)) || (den_floor && o_head < V + 1)) return -2;
+    HeadNormArgs a{o, o_head, w, w_wide, z, ldz, eps, H, V, gate, sub, lambda, post, den_floor};
     llmx_note_launch(LK_HEAD_NORM_GATE);
-    if (out_dtype == LLMX_F32)
-        hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(rows, H), dim3(64), 0, stream, o, w, z, ldz, (float*)out, eps, H, V, gate);
-    else
-        hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3(rows, H), dim3(64), 0, stream, o, w, z, ldz, (bf16_t*)out, eps, H, V, gate);
+    if (out_dtype == LLMX_F32) hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(rows, H), dim3(64), 0, stream, a, (float*)out);
+    else hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3(rows, H), dim3(64), 0, stream, a, (bf16_t*)out);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// A matrix memory with an exponential input gate and a sigmoid forget gate, made ready for the scan above.  Per head and
+// token, from the gates' pre-activations zi, zf (with their biases) and a cap c:
+//     i_t = c tanh(zi / c),  f_t = log sigmoid(c tanh(zf / c)),  m_t = max(f_t + m_(t-1), i_t)       (m starts at 0)
+//     S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,   n_t likewise with k_t alone
+// which is the scan's recurrence with one decay for all of a head's key channels, keys times exp(i_t - m_t), and one more
+// value channel that is always 1 (its column of S is n).  This kernel walks each request's rows in order for m (kept in
+// the request's state slot after the matrix, one float a head) and writes the scan's operands: decay [T, H*D], keys
+// [T, H*D], values [T, H*(V+1)], and exp(-m_t) [T, H], below which the read-out's denominator |n_t . q_t| is not let.
+// One block of 256 threads a (request, head): chunks of 256 rows; a chunk's gates are formed a thread a row, m by every
+// thread alike in row order, the exponentials a thread a row, and the rows are then written a wave a row.
+struct MemoryPrepArgs {
+    const float* pre;        // [T, ld]: the fused projection
+    int ld;
+    int k_col, v_col, i_col, f_col;
+    const float* i_bias;     // [H]
+    const float* f_bias;     // [H]
+    float cap;
+    float* state;
+    long state_stride;
+    int m_off;
+    const int* slot_read;
+    const int* slot_write;
+    const int* entry_rows;
+    float* decay;            // [T, H*D]
+    float* keys;             // [T, H*D]
+    float* values;           // [T, H*(V+1)]
+    float* den_floor;        // [T, H]
+    int H, D, V;
+};
+
+#define MEM_CHUNK 256
+
+__global__ void __launch_bounds__(MEM_CHUNK) memory_prep_kernel(MemoryPrepArgs a) {
+    __shared__ float gi[MEM_CHUNK], gf[MEM_CHUNK], keep[MEM_CHUNK], take[MEM_CHUNK];
+    const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int row0 = a.entry_rows[2 * e], n = a.entry_rows[2 * e + 1];
+    const int H = a.H, D = a.D, V = a.V;
+    float m = a.state[(size_t)a.slot_read[e] * a.state_stride + a.m_off + h];
+    const float bi = a.i_bias[h], bf = a.f_bias[h];
+    for (int c0 = 0; c0 < n; c0 += MEM_CHUNK) {
+        const int rows = min(MEM_CHUNK, n - c0);
+        if (tid < rows) {
+            const float* r = a.pre + (size_t)(row0 + c0 + tid) * a.ld;
+            gi[tid] = a.cap * tanhf((r[a.i_col + h] + bi) / a.cap);
+            const float x = a.cap * tanhf((r[a.f_col + h] + bf) / a.cap);
+            gf[tid] = -(log1pf(expf(-fabsf(x))) + fmaxf(-x, 0.0f));
+        }
+        __syncthreads();
+        float mine_prev = 0.0f, mine_now = 0.0f;
+        for (int t = 0; t < rows; ++t) {        // every thread alike, in row order
+            const float now = fmaxf(gf[t] + m, gi[t]);
+            if (t == tid) {
+                mine_prev = m;
+                mine_now = now;
+            }
+            m = now;
+        }
+        if (tid < rows) {
+            keep[tid] = expf(gf[tid] + mine_prev - mine_now);
+            take[tid] = expf(gi[tid] - mine_now);
+            a.den_floor[(size_t)(row0 + c0 + tid) * H + h] = expf(-mine_now);
+        }
+        __syncthreads();
+        const int wave = tid >> 6, lane = tid & 63;
+        for (int t = wave; t < rows; t += MEM_CHUNK / 64) {
+            const size_t row = (size_t)(row0 + c0 + t);
+            const float* r = a.pre + row * a.ld;
+            const float kp = keep[t], tk = take[t];
+            for (int d = lane; d < D; d += 64) {
+                a.decay[(row * H + h) * D + d] = kp;
+                a.keys[(row * H + h) * D + d] = tk * r[a.k_col + h * D + d];
+            }
+            for (int j = lane; j <= V; j += 64) a.values[(row * H + h) * (V + 1) + j] = j < V ? r[a.v_col + h * V + j] : 1.0f;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) a.state[(size_t)a.slot_write[e] * a.state_stride + a.m_off + h] = m;
+}
+
+extern "C" int llmx_memory_prep(const float* pre, int ld, int k_col, int v_col, int i_col, int f_col, const float* i_bias, const float* f_bias,
+                                float cap, float* state, long state_stride, int m_off, const int* slot_read, const int* slot_write,
+                                const int* entry_rows, float* decay, float* keys, float* values, float* den_floor, int n_entries, int H, int D,
+                                int V, hipStream_t stream) {
+    if (n_entries <= 0) return 0;
+    if (H < 1 || D < 1 || V < 1 || !(cap > 0.0f) || m_off < 0 || m_off + H > state_stride) return -2;
+    MemoryPrepArgs a{pre, ld, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, state, state_stride, m_off, slot_read, slot_write, entry_rows,
+                     decay, keys, values, den_floor, H, D, V};
+    llmx_note_launch(LK_MEMORY_PREP);
+    hipLaunchKernelGGL(memory_prep_kernel, dim3(n_entries, H), dim3(MEM_CHUNK), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
 }

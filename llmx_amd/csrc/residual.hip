@@ -295,7 +295,7 @@ __global__ void __launch_bounds__(256) glu_kernel(const float* __restrict__ pre,
 extern "C" int llmx_act_glu(const float* pre, int ld, const float* row_scale, const float* row_gate, int row_gate_ld, int kind, float limit,
                             void* out, int out_dtype, int rows, int n, hipStream_t stream) {
     if (rows <= 0 || n <= 0) return 0;
-    if (ld < 2 * n || (kind != LLMX_GLU_SILU && kind != LLMX_GLU_CLAMPED) || (kind == LLMX_GLU_CLAMPED && !(limit > 0.0f))) return -2;
+    if (ld < 2 * n || (kind != LLMX_GLU_SILU && kind != LLMX_GLU_CLAMPED && kind != LLMX_GLU_GELU_TANH) || (kind == LLMX_GLU_CLAMPED && !(limit > 0.0f))) return -2;
     llmx_note_launch(LK_ACT_GLU);
     const size_t total = (size_t)rows * n;
     const dim3 grid((unsigned)((total + 255) / 256));

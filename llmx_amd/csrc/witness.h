@@ -78,7 +78,8 @@
     X(ACT_POLYNORM, "act.polynorm")                                                                                       \
     X(ACT_GLU, "act.glu")                                                                                                 \
     X(GATE_HEADS, "gate_heads")                                                                                           \
-    X(RMSNORM_ADD_NORM, "rmsnorm_add_norm")
+    X(RMSNORM_ADD_NORM, "rmsnorm_add_norm")                                                                               \
+    X(MEMORY_PREP, "memory_prep")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

@@ -175,7 +175,7 @@ class Engine:
         self._group_of = [place.get((i, ()), (-1, -1))[0] for i in range(len(needs))]          # cache number -> group (or -1)
         self._index_in_group = [place.get((i, ()), (-1, -1))[1] for i in range(len(needs))]
         self.group_needs = keys
-        groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window) for g, need in enumerate(keys)]
+        groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window, need.keep_first, need.chunk) for g, need in enumerate(keys)]
         groups = [replace(g, n_pages=g.pool_pages(self.kv_tokens, self.max_requests, self.step_tokens)) for g in groups]
         # a model with per-request state steps into a second slot, so that a step that fails leaves the state as it was
         self._stateful = any(isinstance(need, StateNeed) for _, _, need in leaves)

@@ -6,6 +6,7 @@ from . import minimax_m3  # noqa: F401  (registers MiniMaxM3ForCausalLM)
 from . import nenotar  # noqa: F401  (registers Nenotar)
 from . import bonerax  # noqa: F401  (registers Bonerax)
 from . import givozen  # noqa: F401  (registers Givozen)
+from . import salipel  # noqa: F401  (registers Salipel)
 
 __all__ = ["ArchitectureEntry", "architecture_of", "architectures", "assemble", "read_config", "read_model_dir",
            "register_architecture", "unregister_architecture"]

@@ -74,8 +74,8 @@ def _declare(h) -> None:
         "llmx_attention_partial_pad": [],
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, I, P, I, F, P, P, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
-        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P, I, P],
-        "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P, I, P],
+        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, P, I, I, I, I, I, F, P, P, I, P],
+        "llmx_head_norm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, I, P, I, I, I, I, P],
         "llmx_gate_heads": [P, I, P, I, I, I, I, P],
         "llmx_rmsnorm_add_norm": [P, P, P, F, P, F, P, I, P, I, I, P],
         "llmx_add_rows_vector": [P, P, P, I, I, P],
@@ -90,7 +90,8 @@ def _declare(h) -> None:
         "llmx_cast_cols": [P, I, P, I, I, I, P],
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
         "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, I, P],
-        "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, P],
+        "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, I, I, I, F, F, P, P],
+        "llmx_memory_prep": [P, I, I, I, I, I, P, P, F, P, L, I, P, P, P, P, P, P, P, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
@@ -238,19 +239,19 @@ def act_polynorm(z: torch.Tensor, abce: torch.Tensor, eps: float, out: torch.Ten
                                    _dev(out, "out", shape=(rows, n)), _code(out.dtype), rows, n, _stream()), "act_polynorm")
 
 
-GLU_SILU, GLU_CLAMPED = 0, 1
+GLU_SILU, GLU_CLAMPED, GLU_GELU_TANH = 0, 1, 2
 
 
 class Glu:
     """The gated unit of a product's gated epilogue (EPI_SWIGLU) or of `act_glu`.  kind GLU_SILU: silu(gate) * up; GLU_CLAMPED:
-    g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1).  row_scale (float32 [rows of c]; None: 1):
+    g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1); GLU_GELU_TANH: the tanh form of gelu(gate) * up.  row_scale (float32 [rows of c]; None: 1):
     a factor on both pre-activations of a row (a weight on what the product reads, the product being linear); row_gate (a
     float32 view [rows of c, 1], rows possibly strided; None: none): the row's result is multiplied by sigmoid(row_gate)."""
 
     def __init__(self, kind: int = GLU_SILU, limit: float = 0.0, row_scale: Optional[torch.Tensor] = None,
                  row_gate: Optional[torch.Tensor] = None):
-        if kind not in (GLU_SILU, GLU_CLAMPED) or (kind == GLU_CLAMPED and not limit > 0.0):
-            raise KernelError("a gated unit is GLU_SILU or GLU_CLAMPED, the clamped one with a positive limit")
+        if kind not in (GLU_SILU, GLU_CLAMPED, GLU_GELU_TANH) or (kind == GLU_CLAMPED and not limit > 0.0):
+            raise KernelError("a gated unit is GLU_SILU, GLU_CLAMPED or GLU_GELU_TANH, the clamped one with a positive limit")
         self.kind, self.limit, self.row_scale, self.row_gate = int(kind), float(limit), row_scale, row_gate
 
     @property
@@ -694,13 +695,50 @@ def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
 GATE_SIGMOID, GATE_SILU = 0, 1
 
 
-def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor, out: torch.Tensor, eps: float, H: int, V: int, gate: int) -> None:
-    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight * gate(gate_pre[t, h]) for every head's V values; gate is
-    sigmoid or silu of a float32 view [T, H*V]; out in its own type."""
+def head_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], gate_pre: Optional[torch.Tensor], out: torch.Tensor, eps: float, H: int, V: int,
+                   gate: int, minus: Optional[float] = None, post: float = 1.0, den_floor: Optional[torch.Tensor] = None) -> None:
+    """out[t, h] = x / sqrt(mean(x^2) + eps) * weight * gate(gate_pre[t, h]) * post for every head's V values x; gate is
+    sigmoid or silu of a float32 view [T, H*V] (None: no gate); weight float32 [V] (one for all heads), [H*V], or None; out
+    in its own type.  x is o's head [T, H*V]; with `minus` = lambda, o is [T, H*2*V], a head holding two maps, and
+    x = map 1 - lambda * map 2; with `den_floor` (float32 [T, H]), o is [T, H*(V+1)], a head's values followed by their
+    denominator d, and x = values / (max(|d|, den_floor) + 1e-6)."""
     T = o.shape[0]
-    za, ldz = _rows_view(gate_pre, "gate_pre", T, H * V)
-    _check(lib().llmx_head_norm_gate(_dev(o, "o", torch.float32, (T, H * V)), _dev(weight, "weight", torch.float32, (V,)), za, ldz,
-                                     _dev(out, "out", shape=(T, H * V)), _code(out.dtype), float(eps), T, H, V, int(gate), _stream()), "head_norm_gate")
+    o_head = V * (2 if minus is not None else 1) + (1 if den_floor is not None else 0)
+    if minus is not None and den_floor is not None:
+        raise KernelError("head_norm_gate: a second map or a denominator, not both")
+    za, ldz = _rows_view(gate_pre, "gate_pre", T, H * V) if gate_pre is not None else (0, 0)
+    wide = 0
+    if weight is not None:
+        if tuple(weight.shape) not in ((V,), (H * V,)):
+            raise KernelError(f"head_norm_gate: a weight of {V} or {H * V} values, not {tuple(weight.shape)}")
+        wide = 1 if tuple(weight.shape) == (H * V,) and H > 1 else 0
+    _check(lib().llmx_head_norm_gate(_dev(o, "o", torch.float32, (T, H * o_head)), _dev(weight, "weight", torch.float32), za, ldz,
+                                     _dev(out, "out", shape=(T, H * V)), _code(out.dtype), float(eps), T, H, V, int(gate), o_head, wide,
+                                     V if minus is not None else 0, float(minus or 0.0), float(post),
+                                     _dev(den_floor, "den_floor", torch.float32, (T, H)), _stream()), "head_norm_gate")
+
+
+def memory_prep(pre: torch.Tensor, cols: dict, i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float, state: torch.Tensor, m_off: int,
+                slot_read: torch.Tensor, slot_write: torch.Tensor, entry_rows: torch.Tensor, decay: torch.Tensor, keys: torch.Tensor,
+                values: torch.Tensor, den_floor: torch.Tensor, H: int, D: int, V: int) -> None:
+    """A gated matrix memory's rows made ready for `state_scan` (see csrc/linear_state.hip): from the fused projection `pre`
+    [T, ld] with k (H*D), v (H*V) and the two gates' pre-activations (H each) at the columns cols["k"], ["v"], ["i"], ["f"]:
+    i = cap tanh((zi + i_bias) / cap), f = log sigmoid(cap tanh((zf + f_bias) / cap)), the running maximum m = max(f + m, i)
+    of each request (kept at `m_off` of its state slot, one float a head, read at slot_read, written at slot_write);
+    decay [T, H*D] = exp(f + m_before - m), keys [T, H*D] = exp(i - m) k, values [T, H*(V+1)] = v | 1, den_floor [T, H] = exp(-m)."""
+    T, ld = pre.shape
+    n_e = entry_rows.shape[0]
+    if state.dim() != 2 or m_off + H > state.shape[1]:
+        raise KernelError("memory_prep: the state does not hold the running maxima")
+    if max(cols["k"] + H * D, cols["v"] + H * V, cols["i"] + H, cols["f"] + H) > ld:
+        raise KernelError("memory_prep: the projection's rows do not hold the named columns")
+    _check(lib().llmx_memory_prep(_dev(pre, "pre", torch.float32), ld, int(cols["k"]), int(cols["v"]), int(cols["i"]), int(cols["f"]),
+                                  _dev(i_bias, "i_bias", torch.float32, (H,)), _dev(f_bias, "f_bias", torch.float32, (H,)), float(cap),
+                                  _dev(state, "state", torch.float32), state.shape[1], int(m_off), _dev(slot_read, "slot_read", torch.int32, (n_e,)),
+                                  _dev(slot_write, "slot_write", torch.int32, (n_e,)), _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)),
+                                  _dev(decay, "decay", torch.float32, (T, H * D)), _dev(keys, "keys", torch.float32, (T, H * D)),
+                                  _dev(values, "values", torch.float32, (T, H * (V + 1))), _dev(den_floor, "den_floor", torch.float32, (T, H)),
+                                  n_e, H, D, V, _stream()), "memory_prep")
 
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
@@ -766,7 +804,18 @@ def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
     return rows <= NORMED_ROWS_PAY and gemm_f32_can_norm_rows(rows, w)
 
 
-ACT_NONE, ACT_XIELU = 0, 1      # activations a storing product can apply to what it stores
+ACT_NONE, ACT_XIELU, ACT_RELU2 = 0, 1, 2      # activations a storing product can apply to what it stores (RELU2: max(z, 0)^2, no numbers)
+
+
+def _act_args(act, epilogue: int, what: str):
+    """The two values the product kernels take for `act` = (kind, params or None)."""
+    if act is None:
+        return 0, 0
+    if epilogue != EPI_STORE or act[0] not in (ACT_XIELU, ACT_RELU2):
+        raise KernelError(f"{what}: an activation goes with the store epilogue, and xIELU and the squared relu are the ones built")
+    if act[0] == ACT_XIELU:
+        return ACT_XIELU, _dev(act[1], "activation parameters", torch.float32, (2,))
+    return ACT_RELU2, 0
 
 
 def _scratch_now(device):
@@ -789,8 +838,8 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
     `a` may be NormedRows where gemm_takes_normed_rows says so: the product reads bfloat16(norm(x)).
     `scratch(name, shape, dtype)` gives storage that lives as long as the caller's step (a step's workspace): with it,
     products of some tens of rows multiply K's runs in workgroups of their own; the bits are the same either way.
-    `act` = (ACT_XIELU, params): with EPI_STORE, c = activation(a @ w^T), params the activation's numbers on the device
-    (xIELU: float32 (p, q)); the bits of the product followed by the activation's own kernel (act_xielu).
+    `act` = (ACT_XIELU, params) | (ACT_RELU2, None): with EPI_STORE, c = activation(a @ w^T), params the activation's
+    numbers on the device (xIELU: float32 (p, q)); the bits of the product followed by the activation's own kernel (act_xielu).
     `glu`: the gated epilogue's unit (see Glu); None: silu(gate) * up."""
     M, K = a.shape
     if _glu_apart(glu, epilogue):
@@ -801,11 +850,7 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
         act_glu(pre, glu, c)
         return
     glu_args = glu.args(M) if glu is not None and not glu.plain else _NO_GLU
-    act_args = (0, 0)
-    if act is not None:
-        if epilogue != EPI_STORE or act[0] != ACT_XIELU:
-            raise KernelError("gemm: an activation goes with the store epilogue, and xIELU is the one built")
-        act_args = (ACT_XIELU, _dev(act[1], "activation parameters", torch.float32, (2,)))
+    act_args = _act_args(act, epilogue, "gemm")
     N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
@@ -845,8 +890,9 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
                  epilogue: int = EPI_STORE, active: Optional[torch.Tensor] = None, n_active: Optional[torch.Tensor] = None,
                  token_rows: Optional[int] = None, force_generic: bool = False, tile_stats: Optional[torch.Tensor] = None,
-                 glu: Optional["Glu"] = None, scratch=None) -> None:
+                 glu: Optional["Glu"] = None, scratch=None, act=None) -> None:
     """For each group g: rows p in pairs[offsets[g]:offsets[g+1]] get c[p] = a[p // a_div] @ w[g]^T.
+    `act`: as gemm's, for the store epilogue.
 
     With EPI_SWIGLU w[g] holds gate rows then up rows and c[p] = silu(gate) * up.  `active` / `n_active` (from
     moe_align) list the groups that have rows; with them, steps of few token rows (`token_rows`, default the pair
@@ -865,12 +911,13 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         raise KernelError(f"grouped_gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
     n_pairs = pairs.shape[0]
     glu_args = glu.args(c.shape[0]) if glu is not None and not glu.plain else _NO_GLU
+    act_args = _act_args(act, epilogue, "grouped_gemm")
     if c.shape[0] < n_pairs or a.shape[0] * a_div < n_pairs:
         raise KernelError("grouped_gemm: more pairs than rows")
     if token_rows is None:
         token_rows = n_pairs
     if isinstance(a, NormedRows):
-        if active is None or n_active is None or not gemm_can_norm_rows(a.shape[0], w, c.dtype, epilogue, grouped=True):
+        if active is None or n_active is None or act is not None or not gemm_can_norm_rows(a.shape[0], w, c.dtype, epilogue, grouped=True):
             raise KernelError("grouped_gemm: normed rows are not taken for this product")
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
@@ -883,19 +930,19 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, 0, 0, *glu_args, _stream()),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, *act_args, *glu_args, _stream()),
                "grouped_gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                     _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 64, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                     _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0,
-                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, 0, 0, *glu_args, _stream()),
+                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, *act_args, *glu_args, _stream()),
                "grouped_gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    n_pairs, N, K, K, K, N, epilogue, G, _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, 0, 0, *glu_args, _stream()),
+                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *act_args, *glu_args, _stream()),
            "grouped_gemm")
 
 
@@ -928,22 +975,29 @@ def head_norm_rope_kvwrite(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_we
                            cos_sin: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor, tables: torch.Tensor, q_out: torch.Tensor,
                            k_cache: torch.Tensor, v_cache: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, head_dim: int,
                            rotary_dim: int, norm_mode: int, write_kv: bool = True, pairing: int = ROPE_HALVES,
-                           q_scale: Optional[torch.Tensor] = None) -> None:
-    """qknorm_rope_kvwrite for heads that are treated one by one: float32 rows qkv = q (H*D) | k (G*D) | v (G*VD) get the
+                           q_scale: Optional[torch.Tensor] = None, maps: int = 1, values_from_keys: bool = False,
+                           value_norm: bool = False) -> None:
+    """qknorm_rope_kvwrite for heads that are treated one by one: float32 rows qkv = q (H*M*D) | k (G*M*D) | v (G*VD) get the
     projections' biases (`bias`, one vector of that width, or None), every q and k head an RMS norm over its own dims
     with a weight [D] shared by the heads (norm_mode QKNORM_HEAD; QKNORM_NONE: none), then the rotation; k and v go to the
     row's page.  The value width VD is the value cache's and may differ from D.  The rows may be wider than q | k | v (further
-    columns of one fused projection follow v and are left alone).  `q_scale` [H] float32: the rotated q of head h is
-    multiplied by q_scale[h] (a temperature a head on the scores, folded into the query)."""
+    columns of one fused projection follow v and are left alone).  `q_scale` [H*M] float32: the rotated q of head h is
+    multiplied by q_scale[h] (a temperature a head on the scores, folded into the query).  `maps` M > 1: a head has M score
+    maps, each with a query and a key head of its own ([head][map] in q's and k's columns and in the key cache) over one
+    set of values.  `values_from_keys`: the rows hold no v; a value head is its key head as projected (before norm and
+    rotation).  `value_norm`: a value head is divided by its root mean square (eps inside the root) before it is stored."""
     rows = qkv.shape[0]
     n_pages, hk, page_tokens, d = k_cache.shape
     v_dim = v_cache.shape[2]
-    width = n_heads * head_dim + n_kv_heads * head_dim + n_kv_heads * v_dim
+    maps = int(maps)
+    width = n_heads * maps * head_dim + n_kv_heads * maps * head_dim + (0 if values_from_keys else n_kv_heads * v_dim)
     if qkv.dim() != 2 or qkv.shape[1] < width:
         raise KernelError(f"head_norm_rope_kvwrite: rows of {tuple(qkv.shape)} do not hold q | k | v of {width} values")
-    if ((hk, d) != (n_kv_heads, head_dim) or tuple(v_cache.shape) != (n_pages, hk, v_dim, page_tokens) or k_cache.dtype != q_out.dtype
+    if ((hk, d) != (n_kv_heads * maps, head_dim) or tuple(v_cache.shape) != (n_pages, n_kv_heads, v_dim, page_tokens) or k_cache.dtype != q_out.dtype
             or v_cache.dtype != q_out.dtype):
         raise KernelError("head_norm_rope_kvwrite: cache shape or dtype does not fit the heads")
+    if maps < 1 or (values_from_keys and (maps != 1 or v_dim != head_dim)):
+        raise KernelError("head_norm_rope_kvwrite: values taken from the keys are as wide as they, one map a head")
     if rotary_dim % 2 or rotary_dim > head_dim or cos_sin.shape[1] != rotary_dim:
         raise KernelError("head_norm_rope_kvwrite: rotary width does not fit")
     if norm_mode not in (QKNORM_NONE, QKNORM_HEAD):
@@ -954,10 +1008,12 @@ def head_norm_rope_kvwrite(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_we
     _check(lib().llmx_head_norm_rope_kvwrite(
         _dev(qkv, "qkv", torch.float32), _dev(bias, "bias", torch.float32, (width,)), _dev(q_weight, "q_weight"),
         _dev(k_weight, "k_weight"), _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (rows,)),
-        _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32), _dev(q_out, "q_out", shape=(rows, n_heads * head_dim)),
-        _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _code(q_out.dtype), float(eps), rows, n_heads, n_kv_heads, head_dim, v_dim,
+        _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32),
+        _dev(q_out, "q_out", shape=(rows, n_heads * maps * head_dim)),
+        _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _code(q_out.dtype), float(eps), rows, n_heads * maps, n_kv_heads * maps, head_dim, v_dim,
         rotary_dim, norm_mode, page_tokens, tables.shape[1], 1 if write_kv else 0, int(pairing),
-        _dev(q_scale, "q_scale", torch.float32, (n_heads,)), qkv.shape[1], _stream()), "head_norm_rope_kvwrite")
+        _dev(q_scale, "q_scale", torch.float32, (n_heads * maps,)), qkv.shape[1], n_kv_heads, 1 if values_from_keys else 0,
+        1 if value_norm else 0, _stream()), "head_norm_rope_kvwrite")
 
 
 def gate_heads(o: torch.Tensor, gate: torch.Tensor, heads: int) -> None:
@@ -1060,27 +1116,52 @@ def attention_mfma_ok(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bo
     return dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_tokens % 16 == 0
 
 
+class ScoreRules:
+    """What the universal attention kernel does to a row's scores and which keys it sees, beyond the causal rule and a
+    window: keep_first (with a window: the request's first keys stay visible, at their true positions), chunk (a row sees
+    only the keys of its own chunk of positions, counted from the request's start), softcap (score <- softcap tanh(score /
+    softcap)), slopes (float32 [heads]: slopes[h] * (row's position - key's position) is taken off the score), sink (float32
+    [heads]: one more logit a head in the softmax's denominator, without a key or a value), maps (score maps a head over one
+    set of values: q [rows, heads * maps * head_dim], key cache of kv_heads * maps heads, out [rows, heads * maps * v_dim])."""
+
+    def __init__(self, keep_first: int = 0, chunk: int = 0, softcap: float = 0.0, slopes: Optional[torch.Tensor] = None,
+                 sink: Optional[torch.Tensor] = None, maps: int = 1):
+        self.keep_first, self.chunk, self.softcap, self.slopes, self.sink, self.maps = int(keep_first), int(chunk), float(softcap), slopes, sink, int(maps)
+        if self.keep_first < 0 or self.chunk < 0 or self.softcap < 0.0 or self.maps < 1 or (self.keep_first and self.chunk):
+            raise KernelError("attention: keep_first, chunk and softcap are not negative, maps at least 1, and chunks keep no first keys")
+
+    @property
+    def plain(self) -> bool:
+        return not (self.keep_first or self.chunk or self.softcap or self.slopes is not None or self.sink is not None or self.maps != 1)
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
                     tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0,
-                    plan: Optional[AttentionPlan] = None, scratch=None, head_gate: Optional[torch.Tensor] = None) -> None:
+                    plan: Optional[AttentionPlan] = None, scratch=None, head_gate: Optional[torch.Tensor] = None,
+                    rules: Optional[ScoreRules] = None, output_gate: Optional[torch.Tensor] = None) -> None:
     """Causal attention of each row over its request's pages.  With a `plan` (and bfloat16, head_dim a multiple of 16,
     pages of a multiple of 16 tokens, values as wide as keys) the matrix-core kernel runs; `scratch(name, shape, dtype)`
     gives it storage for the partial results of split contexts.  Otherwise the universal kernel runs; it takes values of
     a width of their own (v_cache [pages, kv_heads, v_dim, page_tokens], out [rows, heads * v_dim]).  `head_gate`: a float32
     view [rows, heads] (its rows may be columns of a wider projection): the result of (row, head) is multiplied by the
-    sigmoid of its entry before it is stored, by whichever kernel stores it."""
+    sigmoid of its entry before it is stored, by whichever kernel stores it.  `output_gate`: such a view [rows, heads * v_dim],
+    a logit a value of the result (the universal kernel).  `rules` (ScoreRules): the universal kernel's further score and
+    visibility rules; with several maps `out` may be float32 whatever the cache's type (a later kernel joins the maps)."""
     rows = q.shape[0]
-    n_pages, n_kv_heads, page_tokens, head_dim = k_cache.shape
+    maps = rules.maps if rules is not None else 1
+    n_pages, key_heads, page_tokens, head_dim = k_cache.shape
+    n_kv_heads = v_cache.shape[1]
     v_dim = v_cache.shape[2]
-    if (q.shape[1] != n_heads * head_dim or tuple(out.shape) != (rows, n_heads * v_dim) or q.dtype != k_cache.dtype or out.dtype != q.dtype
-            or v_cache.dtype != q.dtype):
+    if (q.shape[1] != n_heads * maps * head_dim or tuple(out.shape) != (rows, n_heads * maps * v_dim) or q.dtype != k_cache.dtype
+            or (out.dtype != q.dtype and not (maps > 1 and out.dtype == torch.float32)) or v_cache.dtype != q.dtype or key_heads != n_kv_heads * maps):
         raise KernelError("paged_attention: shapes or dtypes do not agree")
     if head_dim > MAX_HEAD_DIM or v_dim > MAX_HEAD_DIM or n_heads % n_kv_heads:
         raise KernelError(f"paged_attention: head_dim {head_dim} or value width {v_dim} above {MAX_HEAD_DIM}, or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
     common = (_dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=(n_pages, n_kv_heads, v_dim, page_tokens)),
               _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32))
     gate_at, gate_ld = _rows_view(head_gate, "head_gate", rows, n_heads) if head_gate is not None else (None, 0)
-    if plan is not None and plan.n_items and v_dim == head_dim and attention_mfma_ok(q.dtype, head_dim, page_tokens):
+    special = (rules is not None and not rules.plain) or output_gate is not None
+    if plan is not None and plan.n_items and v_dim == head_dim and attention_mfma_ok(q.dtype, head_dim, page_tokens) and not special:
         part_o = part_ml = None
         if plan.n_slots:
             if scratch is None:
@@ -1096,8 +1177,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                                _stream()),
                "paged_attention_mfma")
         return
+    gate_wide = 0
+    if output_gate is not None:
+        if head_gate is not None or maps != 1:
+            raise KernelError("paged_attention: one gate, and on one map a head")
+        gate_at, gate_ld = _rows_view(output_gate, "output_gate", rows, n_heads * v_dim)
+        gate_wide = 1
+    r = rules if rules is not None else ScoreRules()
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,
-                                              head_dim, page_tokens, tables.shape[1], int(window), v_dim, gate_at, gate_ld, _stream()), "paged_attention")
+                                              head_dim, page_tokens, tables.shape[1], int(window), v_dim, gate_at, gate_ld, gate_wide,
+                                              r.keep_first, r.chunk, r.maps, r.softcap, _dev(r.slopes, "slopes", torch.float32, (n_heads,)),
+                                              _dev(r.sink, "sink", torch.float32, (n_heads,)), _code(out.dtype), _stream()), "paged_attention")
 
 
 def _parts_args(z: torch.Tensor, parts: Optional[torch.Tensor]):

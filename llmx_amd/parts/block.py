@@ -3,7 +3,8 @@
 "prenorm": x += mixer(norm(x)); x += ffn(norm(x)) with the residual x in float32: the arrangement of
 /root/reference/src/model/arch/minimax_m3.hpp:247-287 (norm, mixer joined into the residual, norm, feed-forward joined).
 "parallel": x += s1 * mixer(norm1(x)) + s2 * ffn(norm2(x)) with both norms of the same x, learned factors s1, s2 a
-coordinate, and an optional per-layer token input after the sum.
+coordinate (or constants), and an optional per-layer token input after the sum; without a second norm both sublayers read
+norm1's rows.
 "outnorm": x += norm1(mixer(x)); x += norm2(ffn(x)): the sublayers read the residual itself and only their results are
 normed.
 "sandwich": x += norm1b(mixer(norm1(x))); x += norm2b(ffn(norm2(x))): a norm on both sides of each sublayer.
@@ -72,16 +73,25 @@ class LayerScale(Part):
         self.weight = tensors.get(self.prefix) if self.optional else tensors[self.prefix]
 
 
+class ConstantScale(Part):
+    """One number on a part's result, a constant of the model.  params: value.  No tensor."""
+    graph_safe = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        self.value = float(params["value"])
+        self.weight = None
+
+
 class ParallelBlock:
     """x += s1 * mixer(norm1(x)) + s2 * ffn(norm2(x)), both of the same x, then an optional token input that reads the
-    new x.  The slots: mixer_norm, mixer, and (both or neither) ffn_norm, ffn; in `extra`: "mixer_scale" and "ffn_scale"
-    (family "scale": a factor a coordinate on each result before the sum, optional) and "token_input" (family
-    "token_input", optional).  Two RMS norms with one eps are one pass over x with two gains."""
+    new x.  The slots: mixer_norm, mixer, ffn_norm, ffn (a feed-forward without a norm of its own reads the mixer's normed
+    rows: one norm for both sublayers); in `extra`: "mixer_scale" and "ffn_scale" (family "scale": a factor a coordinate, or
+    a constant, on each result before the sum, optional) and "token_input" (family "token_input", optional).  Two RMS norms
+    with one eps are one pass over x with two gains."""
     graph_safe = True
 
     def __init__(self, spec: BlockSpec, ctx: BuildContext):
-        if spec.ffn is not None and spec.ffn_norm is None:
-            raise ValueError("parallel block: a feed-forward comes with its norm")
         self.mixer_norm = build_part("norm", spec.mixer_norm, ctx)
         self.mixer = build_part("mixer", spec.mixer, ctx)
         self.ffn_norm = build_part("norm", spec.ffn_norm, ctx) if spec.ffn_norm is not None else None
@@ -104,7 +114,16 @@ class ParallelBlock:
             self.ffn_norm = self.ffn_scale = None
         self.token_input = built.get("token_input")
         a, b = self.mixer_norm, self.ffn_norm
-        self._one_pass = isinstance(a, RMSNorm) and (b is None or (isinstance(b, RMSNorm) and b.eps == a.eps and b.width == a.width))
+        self._shared_norm = self.ffn is not None and self.ffn_norm is None
+        self._one_pass = isinstance(a, RMSNorm) and not self._shared_norm and (b is None or (isinstance(b, RMSNorm) and b.eps == a.eps and b.width == a.width))
+        scales = [s for s in (self.mixer_scale, self.ffn_scale) if s is not None]
+        self._constants = bool(scales) and all(isinstance(s, ConstantScale) for s in scales)
+        if scales and not self._constants and any(isinstance(s, ConstantScale) for s in scales):
+            raise ValueError("parallel block: both scales are constants or both are factors a coordinate")
+        if self._constants and self.token_input is not None:
+            raise ValueError("parallel block: a token input goes with factors a coordinate")
+        if self.ffn is not None and self.ffn.wants_f32_input:
+            self._one_pass = False
 
     def parts(self):
         return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.mixer_scale, self.ffn_scale, self.token_input)
@@ -114,19 +133,28 @@ class ParallelBlock:
         T, E = x.shape
         act = step.act_dtype
         h1 = step.buf("block.h", (T, E), act)
-        h2 = step.buf("block.h2", (T, E), act) if self.ffn is not None else None
-        if self._one_pass:
+        h2 = step.buf("block.h2", (T, E), act) if self.ffn is not None and not self._shared_norm else None
+        # a feed-forward whose router reads unrounded rows gets them from its norm
+        h32 = step.buf("block.h32", (T, E), torch.float32) if self.ffn is not None and self.ffn.wants_f32_input else None
+        if self._shared_norm:
+            self.mixer_norm.forward(step, x, h1, h32)
+            h2 = h1
+        elif self._one_pass:
             ops.rmsnorm_pair(x, self.mixer_norm.weight, self.ffn_norm.weight if h2 is not None else None, self.mixer_norm.eps, h1, h2)
         else:
             self.mixer_norm.forward(step, x, h1)
             if h2 is not None:
-                self.ffn_norm.forward(step, x, h2)
+                self.ffn_norm.forward(step, x, h2, h32)
         y1 = step.buf("block.y1", (T, E), torch.float32)
         self.mixer.forward(step, h1, y1, False, cache)
         y2 = None
         if self.ffn is not None:
             y2 = step.buf("block.y2", (T, E), torch.float32)
-            self.ffn.forward(step, h2, y2, False)
+            self.ffn.forward(step, h2, y2, False, h32)
+        if self._constants:
+            ops.combine_rows(x, y1, self.mixer_scale.value if self.mixer_scale else 1.0, None, y2, self.ffn_scale.value if self.ffn_scale else 1.0,
+                             accumulate=True)
+            return
         copy = step.buf("block.x_act", (T, E), act) if self.token_input is not None else None
         ops.scale_add(x, y1, self.mixer_scale.weight if self.mixer_scale else None, y2, self.ffn_scale.weight if self.ffn_scale else None, copy)
         if self.token_input is not None:
@@ -232,3 +260,4 @@ register("block", "sandwich", SandwichBlock)
 register("block", "outnorm", OutNormBlock)
 register("block", "parallel", ParallelBlock)
 register("scale", "layer_scale", LayerScale)
+register("scale", "constant", ConstantScale)

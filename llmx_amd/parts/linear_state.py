@@ -1,6 +1,6 @@
 """Mixers that carry a float32 matrix state S [key channels D, value channels V] a head from token to token.
 
-Both decay S's rows channel by channel and add an outer product a token; they differ in what is added:
+All decay S's rows (channel by channel, or a head's all alike) and add an outer product a token; they differ in what is added:
     S_t = diag(g_t) S_(t-1) + k_t u_t^T,   o_t = S_t^T q_t
     gated linear attention:  u_t = v_t,                               g_t = sigmoid(z_t)^(1/tau)
     gated delta rule:        u_t = beta_t (v_t - (diag(g_t) S_(t-1))^T k_t),   g_t = exp(-exp(A) softplus(step_t + dt_bias))
@@ -159,5 +159,68 @@ class ChannelDeltaRule(Mixer):
         ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 
+class GatedMatrixMemory(Mixer):
+    """A matrix memory a head with an exponential input gate and a sigmoid forget gate, kept in range by a running maximum m
+    (which starts at 0):
+        i_t = cap tanh((W_i h + b_i) / cap),   f_t = log sigmoid(cap tanh((W_f h + b_f) / cap)),   m_t = max(f_t + m_(t-1), i_t)
+        S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,   n_t the same with k_t alone
+        o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6),   q_t = W_q h dim^-1/2
+    result = W_o (o / rms(o) a head * w * sigmoid(W_g h)), w of all heads' width.  params: hidden, heads, dim, vdim, gate_cap,
+    eps.  Tensors <prefix>q, k, v, g, i, f, i.b, f.b, norm, o.  This is the scan's recurrence with one decay for all of a
+    head's key channels, keys times exp(i_t - m_t) and one more value channel that is always 1, whose column of S is n; the
+    state slot holds that S (in the scan's tiles), then m, one float a head.  Gates, exponentials, the recurrence, its
+    state and the read-out's norm are float32 in both paths."""
+    graph_safe = True
+    steps_between_slots = True
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        p = params
+        self.hidden, self.heads, self.dim, self.vdim = int(p["hidden"]), int(p["heads"]), int(p["dim"]), int(p["vdim"])
+        self.cap, self.eps = float(p["gate_cap"]), float(p["eps"])
+        if min(self.heads, self.dim, self.vdim) < 1 or self.dim > 256 or not self.cap > 0.0:
+            raise ValueError("gated matrix memory: heads, dim (at most 256) and vdim are at least 1 and gate_cap is positive")
+        H, HD, HV = self.heads, self.heads * self.dim, self.heads * self.vdim
+        # the fused in-projection's columns: q | k | v | g | i | f
+        self.cols = {"q": (0, HD), "k": (HD, HD), "v": (2 * HD, HV), "g": (2 * HD + HV, HV), "i": (2 * HD + 2 * HV, H), "f": (2 * HD + 2 * HV + H, H)}
+        self.in_width = 2 * HD + 2 * HV + 2 * H
+        self.state_matrix = ops.state_matrix_size(H, self.dim, self.vdim + 1)
+        self.w_in = self.b_i = self.b_f = self.norm = self.w_o = None
+
+    def cache_need(self):
+        return StateNeed((self.state_matrix + self.heads,), "float32")
+
+    def tensor_specs(self, available):
+        E = self.hidden
+        fused, shape = self.name("in"), (self.in_width, E)
+        specs = [TensorSpec(self.name(n), (w, E), into=(fused, shape, (slice(at, at + w),))) for n, (at, w) in self.cols.items()]
+        return specs + [TensorSpec(self.name("i.b"), (self.heads,), "bias"), TensorSpec(self.name("f.b"), (self.heads,), "bias"),
+                        TensorSpec(self.name("norm"), (self.heads * self.vdim,), "norm"),
+                        TensorSpec(self.name("o"), (E, self.heads * self.vdim))]
+
+    def load(self, tensors):
+        self.w_in = tensors[self.name("in")]
+        self.b_i, self.b_f = tensors[self.name("i.b")], tensors[self.name("f.b")]
+        self.norm, self.w_o = tensors[self.name("norm")], tensors[self.name("o")]
+
+    def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
+        T, H, D, V = step.rows, self.heads, self.dim, self.vdim
+        f32 = torch.float32
+        pre = step.buf("memory.pre", (T, self.in_width), f32)
+        ops.gemm(h, self.w_in, pre, scratch=step.buf)
+        view = lambda n: pre[:, self.cols[n][0]:self.cols[n][0] + self.cols[n][1]]
+        decay, keys = step.buf("memory.decay", (T, H * D), f32), step.buf("memory.keys", (T, H * D), f32)
+        values, floor = step.buf("memory.values", (T, H * (V + 1)), f32), step.buf("memory.floor", (T, H), f32)
+        ops.memory_prep(pre, {n: at for n, (at, _) in self.cols.items()}, self.b_i, self.b_f, self.cap, cache.state, self.state_matrix,
+                        step.entry_held_slots, step.entry_slots, step.entry_rows, decay, keys, values, floor, H, D, V)
+        o = step.buf("memory.o", (T, H * (V + 1)), f32)
+        ops.state_scan(view("q"), keys, values, decay, None, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, o,
+                       float(D) ** -0.5, H, H, D, V + 1, max_rows=step.max_rows_per_entry)
+        gated = step.buf("memory.gated", (T, H * V), step.act_dtype)
+        ops.head_norm_gate(o, self.norm, view("g"), gated, self.eps, H, V, ops.GATE_SIGMOID, den_floor=floor)
+        ops.gemm(gated, self.w_o, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
+
+
+register("mixer", "gated_matrix_memory", GatedMatrixMemory)
 register("mixer", "gated_linear_attention", GatedLinearAttention)
 register("mixer", "channel_delta_rule", ChannelDeltaRule)

@@ -31,7 +31,9 @@ _GLU_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_
 # a shared expert's tensors below the routed feed-forward's prefix
 _EXPERT_NAMES.update({"shared_gate": "shared_expert.gate_proj.weight", "shared_up": "shared_expert.up_proj.weight",
                       "shared_down": "shared_expert.down_proj.weight", "shared_switch": "shared_expert_gate.weight"})
-_UNITS = {"swiglu": ops.GLU_SILU, "clamped_glu": ops.GLU_CLAMPED}
+_UNITS = {"swiglu": ops.GLU_SILU, "clamped_glu": ops.GLU_CLAMPED, "geglu_tanh": ops.GLU_GELU_TANH}
+# units of one product and an activation instead of two products and a gate
+_PLAIN_UNITS = {"relu2": ops.ACT_RELU2}
 
 
 def _names(defaults: dict, given, what: str) -> dict:
@@ -52,7 +54,8 @@ class RoutedExperts(FeedForward):
     "input": sum_j expert_j(w_j h), the weight multiplying what the expert reads; the first product being linear, it is
     applied to both pre-activations before the unit); shared ({intermediate, limit (for clamped_glu), switch (bool)}: an
     expert of the same unit that every row runs, added to the routed sum, times sigmoid(W_switch h) (one number a row)
-    where it has a switch)."""
+    where it has a switch).  unit "relu2": an expert is W_down max(W_up h, 0)^2, with no gate tensor (no shared expert
+    or weight on the input is built for it); "geglu_tanh": the tanh form of gelu(gate) * up."""
     graph_safe = True
 
     wants_f32_input = True
@@ -81,9 +84,10 @@ class RoutedExperts(FeedForward):
         if self.experts > MAX_EXPERTS or self.top_k > MAX_TOP_K:
             raise ValueError(f"routed experts: {self.experts} experts with {self.top_k} picks a token; the routing kernels take at most "
                              f"{MAX_EXPERTS} experts and {MAX_TOP_K} picks")
-        if p.get("unit", "swiglu") not in _UNITS:
-            raise ValueError(f"routed experts: unit {p.get('unit')!r} is not one of {sorted(_UNITS)}")
-        self.unit = _UNITS[p.get("unit", "swiglu")]
+        if p.get("unit", "swiglu") not in _UNITS and p.get("unit") not in _PLAIN_UNITS:
+            raise ValueError(f"routed experts: unit {p.get('unit')!r} is not one of {sorted(list(_UNITS) + list(_PLAIN_UNITS))}")
+        self.plain_unit = _PLAIN_UNITS.get(p.get("unit"))         # None: a gated unit
+        self.unit = _UNITS.get(p.get("unit", "swiglu"), ops.GLU_SILU)
         self.limit = float(p.get("limit") or 0.0)
         if self.unit == ops.GLU_CLAMPED and not self.limit > 0.0:
             raise ValueError("routed experts: the clamped unit needs a positive limit")
@@ -94,6 +98,8 @@ class RoutedExperts(FeedForward):
         self.shared_width = int(shared["intermediate"]) if shared else 0
         self.shared_limit = float(shared.get("limit") or 0.0) if shared else 0.0
         self.shared_switch = bool(shared.get("switch", False)) if shared else False
+        if self.plain_unit is not None and (shared or self.weight_on == "input"):
+            raise ValueError("routed experts: a unit without a gate goes without a shared expert and with the weight on the output")
         if shared and (self.shared_width < 1 or (self.unit == ops.GLU_CLAMPED and not self.shared_limit > 0.0)):
             raise ValueError("routed experts: a shared expert has an inner width of at least 1 and, for the clamped unit, a positive limit")
         self.per_expert = False
@@ -109,6 +115,19 @@ class RoutedExperts(FeedForward):
         if self.use_logit_bias:
             specs.append(TensorSpec(nm("logit_bias"), (X,), "bias"))
         fused = nm("fused_gate_up")
+        if self.plain_unit is not None:        # one product before the activation: the fused tensor holds the up rows alone
+            head, _, tail = self.names["expert_up"].partition("{e}")
+            single = re.compile(re.escape(self.name(head)) + r"\d+" + re.escape(tail) + "$")
+            has_single = any(single.match(n) for n in available)
+            self.per_expert = has_single or (self.files == "per_expert" and fused not in available)
+            down = nm("fused_down")
+            if self.per_expert:
+                for e in range(X):
+                    specs += [TensorSpec(nm("expert_up", e=e), (F, E), into=(fused, (X, F, E), (e,))),
+                              TensorSpec(nm("expert_down", e=e), (E, F), into=(down, (X, E, F), (e,)))]
+            else:
+                specs += [TensorSpec(fused, (X, F, E)), TensorSpec(down, (X, E, F))]
+            return specs
         head, _, tail = self.names["expert_gate"].partition("{e}")
         single = re.compile(re.escape(self.name(head)) + r"\d+" + re.escape(tail) + "$")
         has_single = any(single.match(n) for n in available)
@@ -151,7 +170,7 @@ class RoutedExperts(FeedForward):
                 self.w_switch = tensors[self.name(self.names["shared_switch"])]
 
     def takes_deferred_norm(self, step):
-        if self.shared_width or self.unit != ops.GLU_SILU or self.weight_on == "input":
+        if self.shared_width or self.unit != ops.GLU_SILU or self.weight_on == "input" or self.plain_unit is not None:
             return False           # the shared expert's products and the other gated units read the rows as tensors
         return (ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU, grouped=True)
                 and ops.gemm_f32_takes_normed_rows(step.rows, self.w_router))
@@ -178,9 +197,13 @@ class RoutedExperts(FeedForward):
         step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
         on_input = self.weight_on == "input"
-        glu = ops.Glu(self.unit, self.limit, weights.view(T * k) if on_input else None)
-        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=tile_stats,
-                         glu=glu, scratch=step.buf)
+        if self.plain_unit is not None:
+            ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_STORE, active, n_active, token_rows=T, tile_stats=tile_stats,
+                             act=(self.plain_unit, None))
+        else:
+            glu = ops.Glu(self.unit, self.limit, weights.view(T * k) if on_input else None)
+            ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=tile_stats,
+                             glu=glu, scratch=step.buf)
         y = step.buf("experts.y", (T * k, self.hidden), torch.float32)
         ops.grouped_gemm(act, self.w_down, y, offsets, pairs, 1, ops.EPI_STORE, active, n_active, token_rows=T, tile_stats=tile_stats)
         ops.moe_combine(out, y, ids, None if on_input else weights, accumulate)
@@ -197,8 +220,9 @@ class RoutedExperts(FeedForward):
 
 
 class DenseGLU(FeedForward):
-    """params: hidden, intermediate, names ({role: name below the prefix}).  y = (silu(h.Wg^T) * (h.Wu^T)).Wd^T; tensors
-    gate_proj, up_proj, down_proj (.weight) unless named otherwise."""
+    """params: hidden, intermediate, names ({role: name below the prefix}), unit ("swiglu", the default | "geglu_tanh": the
+    tanh form of gelu on the gate).  y = (silu(h.Wg^T) * (h.Wu^T)).Wd^T; tensors gate_proj, up_proj, down_proj (.weight)
+    unless named otherwise."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
@@ -206,6 +230,9 @@ class DenseGLU(FeedForward):
         self.hidden = int(params["hidden"])
         self.intermediate = int(params["intermediate"])
         self.names = _names(_GLU_NAMES, params.get("names"), "dense GLU")
+        if params.get("unit", "swiglu") not in ("swiglu", "geglu_tanh"):
+            raise ValueError(f"dense GLU: unit {params.get('unit')!r} is not one of ['geglu_tanh', 'swiglu']")
+        self.glu = ops.Glu(_UNITS[params["unit"]]) if params.get("unit", "swiglu") != "swiglu" else None
         self.w_gate_up = self.w_down = None
 
     def tensor_specs(self, available):
@@ -220,11 +247,11 @@ class DenseGLU(FeedForward):
         self.w_down = tensors[self.name(self.names["down"])]
 
     def takes_deferred_norm(self, step):
-        return ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU)
+        return self.glu is None and ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU)
 
     def forward(self, step, h, out, accumulate, h32=None):
         act = step.buf("glu.act", (step.rows, self.intermediate), step.act_dtype)
-        ops.gemm(h, self.w_gate_up, act, ops.EPI_SWIGLU)
+        ops.gemm(h, self.w_gate_up, act, ops.EPI_SWIGLU, glu=self.glu)
         ops.gemm(act, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 

@@ -115,9 +115,13 @@ class CacheTensor:
 class PagedNeed:
     """A mixer that keeps tensors of every position (window None) or of the last `window` positions, in pages.  The
     engine allocates what is listed (one arena a tensor and cache group) and knows nothing else of it; mixers with equal
-    needs share a cache group: one page pool and one block table a request."""
+    needs share a cache group: one page pool and one block table a request.  `keep_first`: under a window the request's
+    first `keep_first` positions are kept as well.  `chunk`: a row reads only positions of its own chunk of `chunk`
+    positions (counted from the request's start), so earlier chunks' pages are given back."""
     tensors: Tuple[CacheTensor, ...]
     window: Optional[int] = None
+    keep_first: int = 0
+    chunk: Optional[int] = None
 
     def __post_init__(self):
         names = [t.name for t in self.tensors]
