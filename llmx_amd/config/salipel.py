@@ -11,7 +11,7 @@ config.json gives every size and every constant that differs between models of t
 
   architecture "Salipel"; vocab; width; norm.eps; residual_mult; layers[]: type, mixer
   (attention: heads, kv_heads, dim, vdim, scale, mask {size};
-   attention_2: heads, kv_heads, dim, vdim, scale, softcap, diff, rot {base, dims, scaling (optional)};
+   attention_2: heads, kv_heads, dim, vdim, scale, softcap (optional), diff, rot {base, dims, scaling (optional)};
    parallel: left {heads, kv_heads, dim, vdim, scale, mask {size, keep_first}, rot {base, dims, scaling {factor, low, high,
    original} (optional)}}, right {heads, dim, vdim, gate_cap}, left_scale, right_scale),
   mlp (null | {kind "dense", ff} | {kind "moe", expert {ff}, router {experts, top, scale}}).
@@ -56,7 +56,7 @@ class DifferenceAttentionConfig:
     dim: int
     vdim: int
     scale: float
-    softcap: float
+    softcap: Optional[float]        # None: the scores are not capped
     diff: float
     rot: Rotation
 
@@ -171,7 +171,7 @@ def _read_mixer(kind: str, m: KeyReader):
         mask.finish((), ARCHITECTURE)
         return out
     if kind == "attention_2":
-        return DifferenceAttentionConfig(softcap=m.real("softcap", positive=True), diff=m.real("diff"), rot=_read_rotation(m), **_heads(m))
+        return DifferenceAttentionConfig(softcap=m.real("softcap", positive=True, default=None), diff=m.real("diff"), rot=_read_rotation(m), **_heads(m))
     left, right = m.child("left"), m.child("right")
     mask = left.child("mask")
     a = WindowAttentionConfig(window=mask.integer("size"), keep_first=mask.integer("keep_first", lo=0, default=0), rot=_read_rotation(left),
@@ -227,7 +227,9 @@ def _layer_json(layer: LayerConfig) -> dict:
         if layer.type == "attention":
             mixer["mask"] = {"size": a.chunk}
         else:
-            mixer.update({"softcap": a.softcap, "diff": a.diff, "rot": _rot_json(a.rot)})
+            mixer.update({"diff": a.diff, "rot": _rot_json(a.rot)})
+            if a.softcap is not None:
+                mixer["softcap"] = a.softcap
     if layer.mlp is None:
         mlp = None
     elif layer.mlp.kind == "dense":

@@ -211,14 +211,14 @@ def difference_attention(h, W, p, cfg, eps):
     root mean square, times (1 - diff), gated."""
     T = h.shape[0]
     H, G, D, V = cfg["heads"], cfg["kv_heads"], cfg["dim"], cfg["vdim"]
-    diff, cap = float(cfg["diff"]), float(cfg["softcap"])
+    diff, cap = float(cfg["diff"]), cfg.get("softcap")
     q = (h @ W[p + "q"].T).reshape(T, H, 2, D)
     k = (h @ W[p + "k"].T).reshape(T, G, 2, D)
     v = (h @ W[p + "v"].T).reshape(T, G, V)
     positions = np.arange(T)
     q = rotate_halves(rms_norm(q, W[p + "q.norm"], eps), positions, cfg["rot"])
     k = rotate_halves(rms_norm(k, W[p + "k.norm"], eps), positions, cfg["rot"])
-    maps = [masked_softmax_attention(q[:, :, a], k[:, :, a], v, cfg["scale"], mask_causal(T), transform=lambda s: cap * np.tanh(s / cap))
+    maps = [masked_softmax_attention(q[:, :, a], k[:, :, a], v, cfg["scale"], mask_causal(T), transform=None if cap is None else (lambda s: cap * np.tanh(s / cap)))
             for a in range(2)]
     o = maps[0] - difference_lambda(W, p, diff) * maps[1]
     o = rms_unit(o, eps) * (1.0 - diff)
