@@ -1,7 +1,7 @@
 """Decode and prefill throughput of MiniMax-M3 at real layer sizes with random weights, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--points 1,64] [--no-sweep] [--no-long]
-    python bench.py --design nenotar|bonerax|givozen [--design-sizes w2048]     (another workload: one design beside the closest model, see --design)
+    python bench.py --design nenotar|bonerax|givozen|salipel [--design-sizes w2048]     (another workload: one design beside the closest model, see --design)
 
 A step is one decode step of the whole batch: B requests, each at a context that reaches C tokens at the last timed
 step, one new token each, logits -> greedy token on the device -> ids read back (the reference's batched `tg`,
@@ -75,7 +75,7 @@ def parse():
     ap.add_argument("--no-generate", action="store_true", help="skip the extra point: the default batch through the scheduler and the sampler")
     ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
     ap.add_argument("--only-long", action="store_true", help="for profiling: run the long-context configuration alone and print its record")
-    ap.add_argument("--design", default=None, help="instead of the default workload: prefill and decode throughput of the named design (nenotar, bonerax, givozen) "
+    ap.add_argument("--design", default=None, help="instead of the default workload: prefill and decode throughput of the named design (nenotar, bonerax, givozen, salipel) "
                     "beside the closest other model at equal size (llmx_amd/tools/design_bench.py); one JSON line of its own")
     ap.add_argument("--design-sizes", default="", help="with --design: the sizes to run, comma separated (default: all)")
     return ap.parse_args()

@@ -1,0 +1,354 @@
+// Paged attention with score and visibility rules on the matrix cores (bfloat16 cache, pages of a multiple of 16 tokens,
+// head_dim a multiple of 8, value width a multiple of 16).
+//
+// What the universal kernel of attention.hip computes a (row, head, map) at a time, for rules the plain causal kernels do
+// not know: a window that also keeps a request's first keys, chunks of positions, a soft cap on the scores, a distance
+// penalty a head, a sink in the softmax's denominator, several score maps a head over one set of values, values of their
+// own width, a gate a value.  A column is a (row, head, map); a wave works on a tile of up to 16 columns: consecutive rows
+// of one request, one head and one map.
+//
+// Keys are grouped in fixed segments of 256 absolute positions, a segment in 8 chunks of 32.  Per column and chunk:
+//   scores^T[key][col] = K_tile[16 keys x D] . Q^T[D x 16 cols]    (A = K, B = Q in registers), two tiles of 16 keys
+//   the rules; an online softmax over the segment's chunks in key order (float32)
+//   o^T[dim][col] += V^T[16 dims x 32 keys] . P^T[32 keys x 16 cols]
+// The value pages are stored transposed, and a chunk's keys are dealt to the rows of its two score tiles (key 8a + 4u + b
+// in row 4a + b of tile u) so that the 8 weights a lane holds belong to 8 consecutive keys: they are the value product's
+// operand as they are.  A chunk or a segment that holds no key a column sees leaves the column's sums as they are, bit
+// for bit, so a column does not see which other columns share its tile.  The segments' (m, l, o) are folded in key order
+// with one formula; a decoded row's long context is shared out over several items that write their segments' (m, l, o),
+// which a second kernel folds in the same order with the same formula: the same bits however the context was shared out.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+#define AR_SEG 256
+#define AR_CHUNKS (AR_SEG / 32)
+#define AR_ITEM_INTS 8
+
+struct RulesArgs {
+    const bf16_t* q;        // [T, heads * maps, D]
+    const bf16_t* k_cache;  // [pages][kv_heads * maps][page_tokens][D]
+    const bf16_t* v_cache;  // [pages][kv_heads][VD][page_tokens]
+    const int* pos;
+    const int* row_entry;
+    const int* tables;
+    const int* items;       // [n][8]: row0, rows, head * maps + map, split, splits, first partial slot (-1: the item stores its result), 0, 0
+    void* out;              // [T, heads * maps * VD], bfloat16 or float32
+    int out_f32;
+    float* part_o;          // [slots][VD]
+    float* part_ml;         // [slots][2]
+    float scale, softcap;
+    int n_heads, n_kv_heads, maps, D, VD, page_tokens, max_blocks;
+    int window, keep_first, chunk;
+    const float* slopes;    // [heads] or null
+    const float* sink;      // [heads] or null
+    const float* gate;      // null, or logits with row stride gate_ld: one a (row, head) or (gate_wide) one a (row, head, value dim)
+    int gate_ld, gate_wide;
+};
+
+// The lowest position, beyond the kept first ones, that a row at position p sees.
+__device__ __forceinline__ int lowest_seen(int p, int window, int chunk) {
+    int lo = 0;
+    if (window > 0 && p - window + 1 > 0) lo = p - window + 1;
+    if (chunk > 0) lo = max(lo, (p / chunk) * chunk);
+    return lo;
+}
+
+// The segments rows at positions first .. last (of one request) see between them: [0, a_end) and [b_begin, b_end).
+struct SegRanges {
+    int a_end, b_begin, b_end;
+    __device__ __forceinline__ int count() const { return a_end + b_end - b_begin; }
+    __device__ __forceinline__ int segment(int ord) const { return ord < a_end ? ord : b_begin + (ord - a_end); }
+};
+__device__ __forceinline__ SegRanges seg_ranges(int first, int last, int window, int keep_first, int chunk) {
+    const int lo = lowest_seen(first, window, chunk);
+    const int kept = min(keep_first, lo);
+    SegRanges r;
+    r.a_end = (kept + AR_SEG - 1) / AR_SEG;
+    r.b_begin = max(lo / AR_SEG, r.a_end);
+    r.b_end = last / AR_SEG + 1;
+    return r;
+}
+
+__device__ __forceinline__ float folded_r(float state, float a, float value, float b) { return fmaf(state, a, value * b); }
+// state (M, L, O) folded with a segment's (m, l, o): the factors on both.  A segment without a seen key changes nothing.
+__device__ __forceinline__ void fold_weights_r(float M, float m, float& a, float& b, float& Mn) {
+    Mn = fmaxf(M, m);
+    if (Mn == -INFINITY) {
+        a = 1.0f;
+        b = 0.0f;
+    } else {
+        a = __expf(M - Mn);
+        b = __expf(m - Mn);
+    }
+}
+
+__device__ __forceinline__ int chunk_key_r(int u, int r) { return 8 * (r >> 2) + 4 * u + (r & 3); }
+
+// The last step of a column: the sink joins the denominator, then result = o / l, times the gate.
+struct Finish {
+    float inv, head_factor;
+    __device__ __forceinline__ Finish(const RulesArgs& a, int row, int h, float M, float L) {
+        float shrink = 1.0f;
+        if (a.sink) {
+            const float sk = a.sink[h];
+            const float top = fmaxf(M, sk);
+            shrink = __expf(M - top);
+            L = L * shrink + __expf(sk - top);
+        }
+        inv = shrink / L;
+        head_factor = (a.gate && !a.gate_wide) ? sigmoid_f(a.gate[(size_t)row * a.gate_ld + h]) : 1.0f;
+    }
+    __device__ __forceinline__ float operator()(const RulesArgs& a, int row, int h, int d, float o) const {
+        float y = o * inv;
+        if (a.gate) y = y * (a.gate_wide ? sigmoid_f(a.gate[(size_t)row * a.gate_ld + (size_t)h * a.VD + d]) : head_factor);
+        return y;
+    }
+};
+
+template <int QS, int DT>
+__global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
+    const int* item = a.items + (size_t)blockIdx.x * AR_ITEM_INTS;
+    const int row0 = item[0], n_rows = item[1], hm = item[2], split = item[3], n_splits = item[4], part_base = item[5];
+    const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
+    const int M = a.maps, D = a.D, VD = a.VD, PT = a.page_tokens;
+    const int h = hm / M, map = hm - h * M;
+    const int kvh = h / (a.n_heads / a.n_kv_heads);
+    const int key_heads = a.n_kv_heads * M, key_head = kvh * M + map;
+    const int qs = (D + 31) / 32, dts = VD / 16;
+    const int p0 = a.pos[row0];
+    const int p_last = p0 + n_rows - 1;
+    const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
+    const bool col_in = c < n_rows;
+    const int p_c = p0 + c;
+    const int lo_c = lowest_seen(p_c, a.window, a.chunk);
+    const int lo_min = lowest_seen(p0, a.window, a.chunk);
+    const int kept_min = min(a.keep_first, lo_min);
+    const float slope = a.slopes ? a.slopes[h] : 0.0f;
+
+    // the columns' queries: lane (c, g) holds dims 32 s + 8 g .. of column c
+    bf16x8_t qf[QS];
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        if (s < qs && col_in && 32 * s + 8 * g + 8 <= D)
+            v = *(const u32x4_t*)(a.q + ((size_t)(row0 + c) * a.n_heads * M + hm) * D + 32 * s + 8 * g);
+        qf[s] = __builtin_bit_cast(bf16x8_t, v);
+    }
+
+    const SegRanges ranges = seg_ranges(p0, p_last, a.window, a.keep_first, a.chunk);
+    const int n_ord = ranges.count();
+    const int per = (n_ord + n_splits - 1) / n_splits;
+    const int ord_begin = split * per, ord_end = min(n_ord, ord_begin + per);
+
+    float Mt = -INFINITY, Lt = 0.0f;
+    f32x4_t Ot[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) Ot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int ord = ord_begin; ord < ord_end; ++ord) {
+        const int seg = ranges.segment(ord);
+        float m = -INFINITY, l = 0.0f;
+        f32x4_t o[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int ch = 0; ch < AR_CHUNKS; ++ch) {
+            const int j0 = seg * AR_SEG + ch * 32;
+            if (j0 > p_last) break;
+            if (j0 + 32 <= lo_min && j0 >= kept_min) continue;      // between the kept keys and the lowest seen one: no column sees any
+            // scores of the chunk's two tiles
+            f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            {
+                const int key0 = j0 + chunk_key_r(0, c), key1 = j0 + chunk_key_r(1, c);
+                const int page0 = key0 <= p_last ? table[key0 / PT] : -1, page1 = key1 <= p_last ? table[key1 / PT] : -1;
+                const bf16_t* k0 = a.k_cache + (((size_t)max(page0, 0) * key_heads + key_head) * PT + key0 % PT) * D + 8 * g;
+                const bf16_t* k1 = a.k_cache + (((size_t)max(page1, 0) * key_heads + key_head) * PT + key1 % PT) * D + 8 * g;
+#pragma unroll
+                for (int s = 0; s < QS; ++s) {
+                    if (s < qs) {
+                        u32x4_t x0 = {0u, 0u, 0u, 0u}, x1 = {0u, 0u, 0u, 0u};
+                        const bool in = 32 * s + 8 * g + 8 <= D;
+                        if (in && page0 >= 0) x0 = *(const u32x4_t*)(k0 + 32 * s);
+                        if (in && page1 >= 0) x1 = *(const u32x4_t*)(k1 + 32 * s);
+                        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x0), qf[s], s0, 0, 0, 0);
+                        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x1), qf[s], s1, 0, 0, 0);
+                    }
+                }
+            }
+            // the lane's 8 scores: keys j0 + 8 g + 0 .. 7 of column c
+            float x[8];
+            float cmax = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int j = j0 + 8 * g + i;
+                float v = (i < 4 ? s0[i] : s1[i - 4]) * a.scale;
+                if (a.softcap > 0.0f) v = a.softcap * tanhf(v / a.softcap);
+                if (a.slopes) v = v - slope * (float)(p_c - j);
+                const bool seen = col_in && j <= p_c && (j >= lo_c || j < a.keep_first);
+                x[i] = seen ? v : -INFINITY;
+                cmax = fmaxf(cmax, x[i]);
+            }
+            cmax = rows_max4(cmax);
+            const float m_new = fmaxf(m, cmax);
+            float corr = 1.0f, w[8], lsum = 0.0f;
+            if (m_new == -INFINITY) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) w[i] = 0.0f;
+            } else {
+                corr = __expf(m - m_new);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    w[i] = __expf(x[i] - m_new);      // 0 for a key that is not seen
+                    lsum += w[i];
+                }
+            }
+            lsum = rows_sum4(lsum);
+            l = fmaf(l, corr, lsum);
+            m = m_new;
+            bf16x8_t pf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pf[i] = (__bf16)w[i];
+            // values: lane (r = c, g) holds dim 16 dt + r, keys j0 + 8 g .. + 7 (one run of a transposed page)
+            const int keyv = j0 + 8 * g;
+            const int pagev = keyv <= p_last ? table[keyv / PT] : -1;
+            const bf16_t* vbase = a.v_cache + (((size_t)max(pagev, 0) * a.n_kv_heads + kvh) * VD + c) * PT + keyv % PT;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                if (dt < dts) {
+                    u32x4_t vv = {0u, 0u, 0u, 0u};
+                    if (pagev >= 0) vv = *(const u32x4_t*)(vbase + (size_t)16 * dt * PT);
+                    o[dt] = f32x4_t{o[dt][0] * corr, o[dt][1] * corr, o[dt][2] * corr, o[dt][3] * corr};
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pf, o[dt], 0, 0, 0);
+                }
+            }
+        }
+        if (part_base >= 0) {       // one column (a decoded row): its segment's sums go out as they are
+            if (c == 0) {
+                const size_t slot = (size_t)part_base + ord;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    if (dt < dts) *(f32x4_t*)(a.part_o + slot * VD + 16 * dt + 4 * g) = o[dt];
+                if (g == 0) {
+                    a.part_ml[2 * slot] = m;
+                    a.part_ml[2 * slot + 1] = l;
+                }
+            }
+        } else {
+            float fa, fb, Mn;
+            fold_weights_r(Mt, m, fa, fb, Mn);
+            Lt = folded_r(Lt, fa, l, fb);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                if (dt < dts)
+                    Ot[dt] = f32x4_t{folded_r(Ot[dt][0], fa, o[dt][0], fb), folded_r(Ot[dt][1], fa, o[dt][1], fb),
+                                     folded_r(Ot[dt][2], fa, o[dt][2], fb), folded_r(Ot[dt][3], fa, o[dt][3], fb)};
+            Mt = Mn;
+        }
+    }
+    if (part_base >= 0 || !col_in) return;
+    const int row = row0 + c;
+    const Finish fin(a, row, h, Mt, Lt);
+    const size_t at = ((size_t)row * a.n_heads * M + hm) * VD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        if (dt < dts) {
+            const int d = 16 * dt + 4 * g;
+            const float y0 = fin(a, row, h, d, Ot[dt][0]), y1 = fin(a, row, h, d + 1, Ot[dt][1]), y2 = fin(a, row, h, d + 2, Ot[dt][2]),
+                        y3 = fin(a, row, h, d + 3, Ot[dt][3]);
+            if (a.out_f32) {
+                *(f32x4_t*)((float*)a.out + at + d) = f32x4_t{y0, y1, y2, y3};
+            } else {
+                bf16_t* dst = (bf16_t*)a.out + at + d;
+                st(dst, y0);
+                st(dst + 1, y1);
+                st(dst + 2, y2);
+                st(dst + 3, y3);
+            }
+        }
+    }
+}
+
+// Folds the segments' sums of a decoded row's column in key order and stores its result: one wave a (row, head, map),
+// lane d owning value dims d, d + 64, ...  merges [n][4]: row, head * maps + map, first partial slot, 0.
+__global__ void __launch_bounds__(64) attention_rules_merge_kernel(RulesArgs a, const int* __restrict__ merges) {
+    const int* mg = merges + (size_t)blockIdx.x * 4;
+    const int row = mg[0], hm = mg[1], base = mg[2];
+    const int lane = threadIdx.x, VD = a.VD, M = a.maps;
+    const int h = hm / M;
+    const int p = a.pos[row];
+    const int n_ord = seg_ranges(p, p, a.window, a.keep_first, a.chunk).count();
+    float Mt = -INFINITY, Lt = 0.0f;
+    float O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int ord = 0; ord < n_ord; ++ord) {
+        const size_t slot = (size_t)base + ord;
+        const float m = a.part_ml[2 * slot], l = a.part_ml[2 * slot + 1];
+        float fa, fb, Mn;
+        fold_weights_r(Mt, m, fa, fb, Mn);
+        Lt = folded_r(Lt, fa, l, fb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int d = lane + 64 * i;
+            if (d < VD) O[i] = folded_r(O[i], fa, a.part_o[slot * VD + d], fb);
+        }
+        Mt = Mn;
+    }
+    const Finish fin(a, row, h, Mt, Lt);
+    const size_t at = ((size_t)row * a.n_heads * M + hm) * VD;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int d = lane + 64 * i;
+        if (d < VD) {
+            const float y = fin(a, row, h, d, O[i]);
+            if (a.out_f32) ((float*)a.out)[at + d] = y;
+            else st((bf16_t*)a.out + at + d, y);
+        }
+    }
+}
+
+extern "C" int llmx_attention_rules_ok(int dtype, int head_dim, int v_dim, int page_tokens) {
+    return dtype == LLMX_BF16 && head_dim >= 8 && head_dim <= 256 && head_dim % 8 == 0 && v_dim >= 16 && v_dim <= 256 && v_dim % 16 == 0 &&
+           page_tokens % 16 == 0;
+}
+
+extern "C" int llmx_attention_rules_segment(void) { return AR_SEG; }
+
+extern "C" int llmx_attention_rules(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry, const int* tables,
+                                    const int* items, int n_items, const int* merges, int n_merges, void* out, int out_f32, float* part_o,
+                                    float* part_ml, float scale, float softcap, int n_heads, int n_kv_heads, int maps, int head_dim, int v_dim,
+                                    int page_tokens, int max_blocks, int window, int keep_first, int chunk, const float* slopes, const float* sink,
+                                    const float* gate, int gate_ld, int gate_wide, hipStream_t stream) {
+    if (n_items <= 0) return 0;
+    if (!llmx_attention_rules_ok(LLMX_BF16, head_dim, v_dim, page_tokens) || maps < 1 || n_heads % n_kv_heads || window < 0 || keep_first < 0 ||
+        chunk < 0 || (n_merges > 0 && (!part_o || !part_ml || !merges)) || (gate && gate_ld < (gate_wide ? n_heads * v_dim : n_heads)))
+        return -2;
+    RulesArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, out, out_f32, part_o, part_ml,
+                scale, softcap, n_heads, n_kv_heads, maps, head_dim, v_dim, page_tokens, max_blocks, window, keep_first, chunk, slopes, sink,
+                gate, gate_ld, gate_wide};
+    llmx_note_launch(LK_ATTENTION_RULES);
+    const int qs = (head_dim + 31) / 32, dts = v_dim / 16;
+#define LLMX_RULES(QS_, DT_) hipLaunchKernelGGL((attention_rules_kernel<QS_, DT_>), dim3(n_items), dim3(64), 0, stream, a)
+    if (qs <= 2) {
+        if (dts <= 4) LLMX_RULES(2, 4);
+        else if (dts <= 8) LLMX_RULES(2, 8);
+        else LLMX_RULES(2, 16);
+    } else if (qs <= 4) {
+        if (dts <= 4) LLMX_RULES(4, 4);
+        else if (dts <= 8) LLMX_RULES(4, 8);
+        else LLMX_RULES(4, 16);
+    } else {
+        if (dts <= 4) LLMX_RULES(8, 4);
+        else if (dts <= 8) LLMX_RULES(8, 8);
+        else LLMX_RULES(8, 16);
+    }
+#undef LLMX_RULES
+    int rc = LLMX_CHECK_LAUNCH();
+    if (rc) return rc;
+    if (n_merges > 0) {
+        llmx_note_launch(LK_ATTENTION_RULES_MERGE);
+        hipLaunchKernelGGL(attention_rules_merge_kernel, dim3(n_merges), dim3(64), 0, stream, a, merges);
+        rc = LLMX_CHECK_LAUNCH();
+    }
+    return rc;
+}

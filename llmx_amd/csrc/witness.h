@@ -79,7 +79,9 @@
     X(ACT_GLU, "act.glu")                                                                                                 \
     X(GATE_HEADS, "gate_heads")                                                                                           \
     X(RMSNORM_ADD_NORM, "rmsnorm_add_norm")                                                                               \
-    X(MEMORY_PREP, "memory_prep")
+    X(MEMORY_PREP, "memory_prep")                                                                                         \
+    X(ATTENTION_RULES, "attention.rules")                                                                                 \
+    X(ATTENTION_RULES_MERGE, "attention.rules_merge")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

@@ -91,6 +91,8 @@ def _declare(h) -> None:
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
         "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, I, P],
         "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, I, I, I, F, F, P, P],
+        "llmx_attention_rules": [P, P, P, P, P, P, P, I, P, I, P, I, P, P, F, F, I, I, I, I, I, I, I, I, I, I, P, P, P, I, I, P],
+        "llmx_attention_rules_ok": [I, I, I, I],
         "llmx_memory_prep": [P, I, I, I, I, I, P, P, F, P, L, I, P, P, P, P, P, P, P, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
@@ -1135,10 +1137,79 @@ class ScoreRules:
         return not (self.keep_first or self.chunk or self.softcap or self.slopes is not None or self.sink is not None or self.maps != 1)
 
 
+class RulesPlan:
+    """Work items of the matrix-core kernel that carries out ScoreRules (csrc/attention_rules.hip) for one step's rows; they
+    hold no positions.  items [n, 8] int32: first row, rows (at most 16, consecutive, of one request), head * maps + map, this
+    item's share and the number of shares its column's segments are dealt into, first slot of the segments' partial sums
+    (-1: the item folds its segments itself and stores the result); merges [n, 4]: row, head * maps + map, first slot."""
+
+    def __init__(self, items, merges, n_slots, device):
+        import numpy as np
+        self.n_items, self.n_merges, self.n_slots = len(items), len(merges), n_slots
+        self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device) if items else None
+        self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 4), device=device) if merges else None
+
+
+RULES_SEGMENT = 256          # keys in a segment of the rules kernel (its AR_SEG)
+RULES_CONTEXT_STEP = 1024    # a decoded row's context is rounded up to this for its plan, so that a growing context keeps its plan (and its graph) for long
+_RULES_PLANS: dict = {}
+
+
+def attention_rules_ok(dtype: torch.dtype, head_dim: int, v_dim: int, page_tokens: int) -> bool:
+    return dtype == torch.bfloat16 and bool(lib().llmx_attention_rules_ok(BF16, int(head_dim), int(v_dim), int(page_tokens)))
+
+
+def rules_plan(row_counts, contexts, n_columns: int, device, window: int = 0, keep_first: int = 0, chunk: int = 0) -> RulesPlan:
+    """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the entry
+    holds after the step; n_columns: heads * maps.  Entries of several rows become tiles of 16 rows a (head, map); a
+    single-row entry (a decoded token) an item a (head, map), its context's segments dealt into shares when the step has few
+    rows.  How the context is shared out changes no result: segments are folded in key order either way."""
+    single = [i for i, n in enumerate(row_counts) if n == 1]
+    rounded = tuple(-(-contexts[i] // RULES_CONTEXT_STEP) * RULES_CONTEXT_STEP if row_counts[i] == 1 else 0 for i in range(len(row_counts)))
+    key = (tuple(row_counts), rounded, n_columns, str(device), window, keep_first, chunk)
+    hit = _RULES_PLANS.get(key)
+    if hit is not None:
+        return hit
+
+    def segments_at_most(context):
+        whole = -(-context // RULES_SEGMENT)
+        if window > 0:
+            whole = min(whole, -(-keep_first // RULES_SEGMENT) + window // RULES_SEGMENT + 2)
+        if chunk > 0:
+            whole = min(whole, chunk // RULES_SEGMENT + 2)
+        return max(1, whole)
+
+    n_splits = {}
+    if single:
+        base = len(single) * n_columns
+        for i in single:
+            n_splits[i] = max(1, min(segments_at_most(rounded[i]), ATTENTION_TARGET_WAVES // base))
+    items, merges, slots, row = [], [], 0, 0
+    for i, n in enumerate(row_counts):
+        if n == 1 and n_splits[i] > 1:
+            cap = segments_at_most(rounded[i])
+            for hm in range(n_columns):
+                for s in range(n_splits[i]):
+                    items.append([row, 1, hm, s, n_splits[i], slots, 0, 0])
+                merges.append([row, hm, slots, 0])
+                slots += cap
+        else:
+            for r0 in range(0, n, 16):
+                for hm in range(n_columns):
+                    items.append([row + r0, min(16, n - r0), hm, 0, 1, -1, 0, 0])
+        row += n
+    plan = RulesPlan(items, merges, slots, device)
+    if len(_RULES_PLANS) > 256:
+        _RULES_PLANS.clear()
+    _RULES_PLANS[key] = plan
+    return plan
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
                     tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0,
                     plan: Optional[AttentionPlan] = None, scratch=None, head_gate: Optional[torch.Tensor] = None,
-                    rules: Optional[ScoreRules] = None, output_gate: Optional[torch.Tensor] = None) -> None:
+                    rules: Optional[ScoreRules] = None, output_gate: Optional[torch.Tensor] = None,
+                    rules_plan: Optional[RulesPlan] = None) -> None:
     """Causal attention of each row over its request's pages.  With a `plan` (and bfloat16, head_dim a multiple of 16,
     pages of a multiple of 16 tokens, values as wide as keys) the matrix-core kernel runs; `scratch(name, shape, dtype)`
     gives it storage for the partial results of split contexts.  Otherwise the universal kernel runs; it takes values of
@@ -1146,7 +1217,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     view [rows, heads] (its rows may be columns of a wider projection): the result of (row, head) is multiplied by the
     sigmoid of its entry before it is stored, by whichever kernel stores it.  `output_gate`: such a view [rows, heads * v_dim],
     a logit a value of the result (the universal kernel).  `rules` (ScoreRules): the universal kernel's further score and
-    visibility rules; with several maps `out` may be float32 whatever the cache's type (a later kernel joins the maps)."""
+    visibility rules; with several maps `out` may be float32 whatever the cache's type (a later kernel joins the maps).
+    `rules_plan` (from `rules_plan`, for this step's rows and these rules): where the sizes allow (`attention_rules_ok`) the
+    matrix-core kernel for rules runs instead of the universal one."""
     rows = q.shape[0]
     maps = rules.maps if rules is not None else 1
     n_pages, key_heads, page_tokens, head_dim = k_cache.shape
@@ -1184,6 +1257,21 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         gate_at, gate_ld = _rows_view(output_gate, "output_gate", rows, n_heads * v_dim)
         gate_wide = 1
     r = rules if rules is not None else ScoreRules()
+    if rules_plan is not None and rules_plan.n_items and attention_rules_ok(q.dtype, head_dim, v_dim, page_tokens):
+        part_o = part_ml = None
+        if rules_plan.n_slots:
+            if scratch is None:
+                scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=q.device)
+            part_o = scratch("attention.rules_part_o", (rules_plan.n_slots, v_dim), torch.float32)
+            part_ml = scratch("attention.rules_part_ml", (rules_plan.n_slots, 2), torch.float32)
+        _check(lib().llmx_attention_rules(*common, _dev(rules_plan.items, "items", torch.int32), rules_plan.n_items,
+                                          _dev(rules_plan.merges, "merges", torch.int32), rules_plan.n_merges, _dev(out, "out"),
+                                          1 if out.dtype == torch.float32 else 0, _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale),
+                                          r.softcap, n_heads, n_kv_heads, r.maps, head_dim, v_dim, page_tokens, tables.shape[1], int(window),
+                                          r.keep_first, r.chunk, _dev(r.slopes, "slopes", torch.float32, (n_heads,)),
+                                          _dev(r.sink, "sink", torch.float32, (n_heads,)), gate_at, gate_ld, gate_wide, _stream()),
+               "attention_rules")
+        return
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,
                                               head_dim, page_tokens, tables.shape[1], int(window), v_dim, gate_at, gate_ld, gate_wide,
                                               r.keep_first, r.chunk, r.maps, r.softcap, _dev(r.slopes, "slopes", torch.float32, (n_heads,)),

@@ -212,9 +212,22 @@ class Attention(Mixer):
                            lambda: ops.attention_plan([e.n for e in step.entries], [e.past + e.n for e in step.entries], self.heads,
                                                       self.kv_heads, step.device, window))
 
+    def _rules_plan(self, step):
+        """The work items of the matrix-core kernel for rules, made once a step and shared by every layer with the same
+        columns and rules."""
+        window = int(self.window or 0)
+        return step.shared(("attention.rules_plan", self.heads * self.maps, window, self.keep_first, self.chunk),
+                           lambda: ops.rules_plan([e.n for e in step.entries], [e.past + e.n for e in step.entries], self.heads * self.maps,
+                                                  step.device, window, self.keep_first, self.chunk))
+
+    def _rules_mfma(self, act, page_tokens):
+        return self.special and ops.attention_rules_ok(act, self.head_dim, self.v_dim, page_tokens)
+
     def graph_key(self, step):
         # a recorded step holds the plan's addresses and launch sizes; the universal kernel has no plan
         page = self.ctx.page_tokens
+        if page and self._rules_mfma(step.act_dtype, page):
+            return self._rules_plan(step)
         return self._plan(step) if page and self._mfma(step.act_dtype, page) else None
 
     def _mfma(self, act, page_tokens):
@@ -240,18 +253,19 @@ class Attention(Mixer):
                                     pairing=self.pairing)
         o = step.buf("attention.out", (T, self.o_width), act)
         plan = self._plan(step) if self._mfma(act, cache.k.shape[2]) else None
+        by_rules = self._rules_plan(step) if self._rules_mfma(act, cache.k.shape[2]) else None
         if self.difference:
             # both maps' results in float32, then their difference, its norm a head and the gate in one kernel
             both = step.buf("attention.maps", (T, self.maps * self.o_width), torch.float32)
             ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, both, self.scale, self.heads,
-                                window=int(self.window or 0), rules=self.rules)
+                                window=int(self.window or 0), rules=self.rules, rules_plan=by_rules, scratch=step.buf)
             ops.head_norm_gate(both, None, qkv[:, qkv_width:] if self.output_gate else None, o, self.eps, self.heads, self.v_dim,
                                ops.GATE_SIGMOID, minus=self.lam, post=1.0 - self.diff)
         else:
             ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
                                 window=int(self.window or 0), plan=plan, scratch=step.buf,
                                 head_gate=qkv[:, qkv_width:] if self.head_gate else None,      # the gate a head, where the result is stored
-                                rules=self.rules, output_gate=qkv[:, qkv_width:] if self.output_gate else None)
+                                rules=self.rules, output_gate=qkv[:, qkv_width:] if self.output_gate else None, rules_plan=by_rules)
         if self.b_o is not None and add_output_bias:
             y = step.buf("attention.projected", (T, self.hidden), torch.float32)
             ops.gemm(o, self.wo, y, scratch=step.buf)

@@ -9,6 +9,10 @@ routed clamped-unit experts with a shared expert, two of them run twice; attenti
 a head) and a MiniMax-M3 with as many layers as the Givozen has layer runs and the same width, heads, head width, experts,
 picks and expert width.  A repeated layer's weights count each time they run.
 
+`python bench.py --design salipel` does the same for a Salipel (layers in turn: two score maps a head with a dense gated
+unit, the same with routed squared-relu experts, windowed attention that keeps the first tokens beside a gated matrix memory,
+attention in chunks with routed experts) and a MiniMax-M3 of the same width, layers, heads, experts, picks and expert width.
+
 `python bench.py --design nenotar` measures, at sizes that resemble a real model's layers, a Nenotar (latent attention
 and minGRU layers in turn, each with a dense xIELU feed-forward and a per-layer token input) and a MiniMax-M3 of the
 same width, layers, heads and vocabulary whose routed experts hold the same active weights a token: one 2,048-token
@@ -141,6 +145,81 @@ def givozen_work(cfg, rows: int):
     return used, read
 
 
+# name -> (width, layers, heads, kv heads, window, chunk, memory heads (of 128 x 128), dense ff, experts, picks, expert ff, vocab)
+SALIPEL_SIZES = {
+    "w2048": (2048, 8, 16, 4, 1024, 1024, 4, 8192, 8, 2, 2048, 32768),
+    "w4096": (4096, 4, 32, 8, 1024, 1024, 8, 16384, 8, 2, 4096, 32768),
+    "w256": (256, 4, 2, 1, 64, 48, 1, 768, 4, 2, 128, 1024),
+}
+
+
+def salipel_config(width, layers, heads, kv_heads, window, chunk, mem_heads, dense_ff, experts, top, ff, vocab):
+    from llmx_amd.config.givozen import WavelengthScaling
+    from llmx_amd.config.salipel import (ChunkAttentionConfig, DifferenceAttentionConfig, LayerConfig, MemoryConfig, MLPConfig, ParallelConfig,
+                                         Rotation, SalipelConfig, WindowAttentionConfig)
+    rot = Rotation(1e6, 64, WavelengthScaling(8.0, 1.0, 4.0, 8192.0))
+    two = DifferenceAttentionConfig(heads=heads, kv_heads=kv_heads, dim=64, vdim=128, scale=64 ** -0.5, softcap=50.0, diff=0.3, rot=rot)
+    side = ParallelConfig(WindowAttentionConfig(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, window=window, keep_first=4, rot=rot),
+                          MemoryConfig(heads=mem_heads, dim=128, vdim=128, gate_cap=15.0), 1.0, 0.5)
+    chunks = ChunkAttentionConfig(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, chunk=chunk)
+    dense, moe = MLPConfig("dense", dense_ff), MLPConfig("moe", ff, experts=experts, top=top, scale=2.0)
+    kinds = [("attention_2", two, dense), ("attention_2", two, moe), ("parallel", side, dense), ("attention", chunks, moe)]
+    return SalipelConfig(vocab=vocab, width=width, norm_eps=1e-6, residual_mult=0.7, layers=tuple(LayerConfig(*kinds[i % 4]) for i in range(layers)))
+
+
+def salipel_closest(width, layers, heads, kv_heads, window, chunk, mem_heads, dense_ff, experts, top, ff, vocab):
+    """MiniMax-M3 of the same width, layers, heads, head width, experts, picks and expert width."""
+    return bonerax_closest(width, layers, heads, kv_heads, window, mem_heads, experts, top, ff, vocab)
+
+
+def salipel_work(cfg, rows: int):
+    """(weights a step of `rows` rows multiplies a row by, weights it must read), both in elements; of routed experts a row
+    uses `top` and a step reads at most rows x top."""
+    used = read = 0.0
+    E = cfg.width
+    for layer in cfg.layers:
+        m = layer.mixer
+        if layer.type == "attention":
+            mix = E * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + m.heads * m.vdim * E
+        elif layer.type == "attention_2":
+            mix = E * (2 * m.heads * m.dim + m.kv_heads * (2 * m.dim + m.vdim) + m.heads * m.vdim) + m.heads * m.vdim * E
+        else:
+            a, b = m.left, m.right
+            mix = E * (a.heads * a.dim + a.kv_heads * a.dim + a.heads * a.vdim) + a.heads * a.vdim * E
+            mix += E * (2 * b.heads * b.dim + 2 * b.heads * b.vdim + 2 * b.heads) + b.heads * b.vdim * E
+        used += mix
+        read += mix
+        mlp = layer.mlp
+        if mlp is None:
+            continue
+        if mlp.kind == "dense":
+            used += 3 * E * mlp.ff
+            read += 3 * E * mlp.ff
+        else:
+            used += E * mlp.experts + mlp.top * 2 * E * mlp.ff
+            read += E * mlp.experts + min(mlp.experts, rows * mlp.top) * 2 * E * mlp.ff
+    return used, read
+
+
+def salipel_mixing_flops(cfg, T: int) -> float:
+    """Multiply-adds x 2 of the mixers' own work over a T-token prompt: scores and value products over the keys a row sees
+    (twice the scores for two maps, and two value products), and the matrix memory's decay, outer product and read-out."""
+    total = 0.0
+    for layer in cfg.layers:
+        m = layer.mixer
+        if layer.type == "attention":
+            keys = sum(t % m.chunk + 1 for t in range(T))
+            total += 2.0 * m.heads * (m.dim + m.vdim) * keys
+        elif layer.type == "attention_2":
+            total += 2.0 * m.heads * 2 * (m.dim + m.vdim) * T * (T + 1) / 2
+        else:
+            a, b = m.left, m.right
+            keys = sum(min(t + 1, a.window) + min(a.keep_first, max(0, t + 1 - a.window)) for t in range(T))
+            total += 2.0 * a.heads * (a.dim + a.vdim) * keys
+            total += T * b.heads * b.dim * (b.vdim + 1) * 5.0
+    return total
+
+
 def _layer_mixers(layer):
     """(windowed attention or None, [recurrences as (heads, dim, vdim, delta?)]) of a Bonerax layer."""
     m = layer.mixer
@@ -168,7 +247,9 @@ def cache_bytes_read(engine, context: float) -> float:
     a windowed group's keys and values only as far as the window reaches."""
     total = 0.0
     for need, arenas in zip(engine.group_needs, engine._paged):
-        tokens = min(context, need.window) if need.window else context
+        tokens = min(context, need.window + getattr(need, "keep_first", 0)) if need.window else context
+        if getattr(need, "chunk", None):
+            tokens = min(tokens, need.chunk / 2.0)      # a decoded row sits anywhere in its chunk
         total += tokens * sum(t.shape[0] * (t.numel() // (t.shape[0] * t.shape[1]) // engine.page_tokens) * t.element_size() for t in arenas.values())
     return total + 2 * sum(t[0].numel() * t.element_size() for t in engine._state)
 
@@ -188,6 +269,9 @@ def prompt_flops(engine, T) -> float:
     elif cfg.architecture == "Givozen":
         dense = 2.0 * T * givozen_work(cfg, T)[0] + 2.0 * vocab * engine.spec.hidden_size
         attn = sum(2.0 * cfg.layers[i].mixer.heads * (cfg.layers[i].mixer.dim + cfg.layers[i].mixer.vdim) * T * (T + 1) / 2 for i, _, _ in cfg.passes())
+    elif cfg.architecture == "Salipel":
+        dense = 2.0 * T * salipel_work(cfg, T)[0] + 2.0 * vocab * engine.spec.hidden_size
+        attn = salipel_mixing_flops(cfg, T)
     elif cfg.architecture == "Bonerax":
         attn = 0.0
         for layer in cfg.layers:
@@ -272,6 +356,8 @@ def measure(engine, torch, steps, warmup):
         side = getattr(cfg, "token_side_dim", None) or 0
         need -= 2 * vocab * side * (len(cfg.layers) if side else 0)     # of the token table a step reads its rows only
         need -= 2 * vocab * engine.spec.hidden_size                     # and of the embedding
+        if cfg.architecture == "Salipel":
+            need = 2 * (salipel_work(cfg, batch)[1] + vocab * engine.spec.hidden_size) + batch * cache_bytes_read(engine, CONTEXT - steps / 2)
         if cfg.architecture == "Givozen":       # weights by layer run; the head is the embedding's table, read whole
             need = 2 * (givozen_work(cfg, batch)[1] + vocab * engine.spec.hidden_size) + batch * cache_bytes_read(engine, CONTEXT - steps / 2)
         rec.update({f"decode_b{batch}_tok_s": round(batch / dt, 2), f"decode_b{batch}_ms": round(dt * 1e3, 4),
@@ -283,6 +369,7 @@ DESIGNS = {
     "nenotar": ("Nenotar", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", SIZES, nenotar_config, closest_config),
     "bonerax": ("Bonerax", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", BONERAX_SIZES, bonerax_config, bonerax_closest),
     "givozen": ("Givozen", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", GIVOZEN_SIZES, givozen_config, givozen_closest),
+    "salipel": ("Salipel", "MiniMax-M3 (GQA attention, routed SwiGLU experts)", SALIPEL_SIZES, salipel_config, salipel_closest),
 }
 
 

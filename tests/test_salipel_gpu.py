@@ -162,13 +162,17 @@ def _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, sharp=None, 
         o.head_norm_rope_kvwrite(rows, None, qw, kw, cos_sin, pos, ent, tables, q, kc, vc, eps, H, G, D, R, o.QKNORM_HEAD if normed else o.QKNORM_NONE,
                                  pairing=o.ROPE_HALVES, maps=M, values_from_keys=kind == "window", value_norm=kind == "chunks")
         part = torch.empty(n, H * V, device="cuda", dtype=dtype)
+        # where the sizes allow, the matrix-core kernel for rules (its work items made for this launch's rows)
+        plan = None
+        if o.attention_rules_ok(dtype, D, V, page):
+            plan = o.rules_plan([n], [b], H * M, torch.device("cuda"), window, rules.keep_first, rules.chunk)
         if kind == "two_maps":
             both = torch.empty(n, H * 2 * V, device="cuda", dtype=torch.float32)
-            o.paged_attention(q, kc, vc, pos, ent, tables, both, scale, H, rules=rules)
+            o.paged_attention(q, kc, vc, pos, ent, tables, both, scale, H, rules=rules, rules_plan=plan)
             o.head_norm_gate(both, None, rows[:, width:], part, eps, H, V, o.GATE_SIGMOID, minus=plain.difference_lambda(W, "p.", rule[1]), post=1.0 - rule[1])
         else:
             o.paged_attention(q, kc, vc, pos, ent, tables, part, scale, H, window=window, rules=rules,
-                              output_gate=rows[:, width:] if kind == "window" else None)
+                              output_gate=rows[:, width:] if kind == "window" else None, rules_plan=plan)
         out[a:b] = part
     return out.float().cpu(), torch.as_tensor(want)
 
@@ -179,9 +183,10 @@ ATT_TOL = {torch.float32: 2e-5, torch.bfloat16: 4e-2}
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
 @pytest.mark.parametrize("case", [
     ("window", 4, 2, 32, 32, 16, 16, 150, (24, 3)), ("window", 3, 1, 10, 10, 6, 4, 90, (5, 0)), ("window", 2, 2, 128, 128, 64, 16, 200, (70, 9)),
-    ("window", 4, 4, 16, 16, 16, 16, 60, (300, 8)), ("window", 2, 1, 24, 24, 0, 8, 70, (1, 5)),
+    ("window", 4, 4, 16, 16, 16, 16, 60, (300, 8)), ("window", 2, 1, 24, 24, 0, 8, 70, (1, 5)), ("window", 2, 1, 64, 64, 32, 16, 1300, (700, 300)),
     ("chunks", 4, 1, 16, 32, 0, 16, 150, 40), ("chunks", 3, 3, 10, 6, 0, 4, 60, 7), ("chunks", 8, 2, 64, 64, 0, 16, 200, 64), ("chunks", 2, 1, 48, 8, 0, 16, 40, 1),
     ("two_maps", 4, 2, 32, 64, 16, 16, 150, (30.0, 0.25)), ("two_maps", 3, 1, 10, 14, 10, 4, 70, (1.5, 0.5)), ("two_maps", 2, 2, 64, 128, 0, 16, 130, (None, 0.3)),
+    ("two_maps", 2, 1, 48, 96, 16, 16, 1100, (20.0, 0.2)), ("chunks", 2, 1, 32, 48, 0, 16, 1200, 600),
 ], ids=lambda c: f"{c[0]}-{c[1]}x{c[3]}")
 def test_the_three_attention_forms_over_shuffled_pages(dtype, case):
     kind, H, G, D, V, R, page, length, rule = case
@@ -459,9 +464,9 @@ def test_windows_and_chunks_give_pages_back_while_a_request_runs():
 
 
 def test_which_kernels_a_serving_step_takes():
-    """The launch witness: a bfloat16 step at sizes the matrix cores take (configuration A) runs the design's kernels and
-    the matrix-core products; the design's attention forms are the universal kernel's; a float32 engine launches no
-    bfloat16 product."""
+    """The launch witness: a bfloat16 step at sizes the matrix cores take (configuration A) runs the design's kernels, the
+    matrix-core products and the matrix-core attention for rules (a decoded row's context shared out and merged), never
+    the universal ones; a float32 engine runs the universal attention and launches no bfloat16 product."""
     from llmx_amd.engine import StepEntry
     o = ops()
     tokens = tokens_for("A", 70, 2)
@@ -474,19 +479,20 @@ def test_which_kernels_a_serving_step_takes():
             engine.step([entry])
             for name, count in o.take_launches().items():
                 seen[name] = seen.get(name, 0) + count
-        for name in ("head_norm_rope_kvwrite", "attention.generic", "memory_prep", "state_scan", "head_norm_gate", "combine_rows", "rmsnorm",
+        for name in ("head_norm_rope_kvwrite", "memory_prep", "state_scan", "head_norm_gate", "combine_rows", "rmsnorm",
                      "moe_combine", "route_topk"):
             assert seen.get(name), f"{dtype}: no launch of {name} ({sorted(seen)})"
-        assert seen["attention.generic"] == 2 * 4 and seen["memory_prep"] == 2 and seen["state_scan"] == 2
+        assert seen["attention.rules" if dtype == "bfloat16" else "attention.generic"] == 2 * 4 and seen["memory_prep"] == 2 and seen["state_scan"] == 2
         assert seen["head_norm_gate"] == 2 * 3                  # two layers of two maps and the memory's read-out
         assert seen["combine_rows"] == 2 * (4 + 1)              # every layer's join, and the side-by-side mixer's
         assert seen["rmsnorm"] >= 2 * 4                         # one norm a layer (and the model's, where a step wants rows)
         assert "act.glu" not in seen and "gate_heads" not in seen       # the units run in the products' epilogues
         if dtype == "bfloat16":
-            assert not any(n.startswith("gemm_generic") for n in seen), sorted(seen)
+            assert not any(n.startswith(("gemm_generic", "attention.generic")) for n in seen), sorted(seen)
+            assert seen.get("attention.rules_merge")
             assert any(n.startswith("gemm_skinny") or n.startswith("gemm_tile") for n in seen)
         else:
-            assert not any(n.startswith(("gemm_skinny", "gemm_tile")) for n in seen), sorted(seen)
+            assert not any(n.startswith(("gemm_skinny", "gemm_tile", "attention.rules")) for n in seen), sorted(seen)
 
 
 def test_a_failed_step_leaves_pages_and_states_as_they_were():
