@@ -5,9 +5,9 @@
 // not know: a window that also keeps a request's first keys, chunks of positions, a soft cap on the scores, a distance
 // penalty a head, a sink in the softmax's denominator, several score maps a head over one set of values, values of their
 // own width, a gate a value.  A column is a (row, head, map); a wave works on a tile of up to 16 columns: consecutive rows
-// of one request, one head and one map.
+// of one request, one map, and the query heads that read one key/value head (see the kernel).
 //
-// Keys are grouped in fixed segments of 256 absolute positions, a segment in 8 chunks of 32.  Per column and chunk:
+// Keys are grouped in fixed segments of 128 absolute positions, a segment in 4 chunks of 32.  Per column and chunk:
 //   scores^T[key][col] = K_tile[16 keys x D] . Q^T[D x 16 cols]    (A = K, B = Q in registers), two tiles of 16 keys
 //   the rules; an online softmax over the segment's chunks in key order (float32)
 //   o^T[dim][col] += V^T[16 dims x 32 keys] . P^T[32 keys x 16 cols]
@@ -23,9 +23,10 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-#define AR_SEG 256
+#define AR_SEG 128
 #define AR_CHUNKS (AR_SEG / 32)
 #define AR_ITEM_INTS 8
+#define AR_MERGE_MAX 256    // segments whose maxima and sums the merge holds at a time
 
 struct RulesArgs {
     const bf16_t* q;        // [T, heads * maps, D]
@@ -34,7 +35,7 @@ struct RulesArgs {
     const int* pos;
     const int* row_entry;
     const int* tables;
-    const int* items;       // [n][8]: row0, rows, head * maps + map, split, splits, first partial slot (-1: the item stores its result), 0, 0
+    const int* items;       // [n][8]: row0, rows, first head, split, splits, first partial slot (-1: the item stores its result), map, 0
     void* out;              // [T, heads * maps * VD], bfloat16 or float32
     int out_f32;
     float* part_o;          // [slots][VD]
@@ -46,6 +47,7 @@ struct RulesArgs {
     const float* sink;      // [heads] or null
     const float* gate;      // null, or logits with row stride gate_ld: one a (row, head) or (gate_wide) one a (row, head, value dim)
     int gate_ld, gate_wide;
+    int hpc;                // query heads of a tile's columns: those of one key/value head where their number divides 16, else 1
 };
 
 // The lowest position, beyond the kept first ones, that a row at position p sees.
@@ -85,6 +87,10 @@ __device__ __forceinline__ void fold_weights_r(float M, float m, float& a, float
     }
 }
 
+// tanh as 1 - 2 / (e^2x + 1) with the fast exponential: a few instructions where the library's routine takes tens; its
+// absolute error of about 1e-7 (times the cap, on a score) is far below what the bfloat16 operands carry.
+__device__ __forceinline__ float tanh_fast(float x) { return 1.0f - __fdividef(2.0f, __expf(2.0f * x) + 1.0f); }
+
 __device__ __forceinline__ int chunk_key_r(int u, int r) { return 8 * (r >> 2) + 4 * u + (r & 3); }
 
 // The last step of a column: the sink joins the denominator, then result = o / l, times the gate.
@@ -108,25 +114,32 @@ struct Finish {
     }
 };
 
+// A tile's 16 columns are `hpc` query heads (those that read one key/value head, where their number divides 16; else one
+// head) for each of 16 / hpc consecutive rows: column c is row c / hpc of the tile, head h0 + c % hpc.  The keys and values
+// a chunk brings are then multiplied for all of a key/value head's query heads at once.
+// A segment's page ids are read once (lane i holds the i-th page the segment touches) and handed round by lane index; the
+// next chunk's keys and values are asked for before this chunk's are multiplied.
 template <int QS, int DT>
 __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
     const int* item = a.items + (size_t)blockIdx.x * AR_ITEM_INTS;
-    const int row0 = item[0], n_rows = item[1], hm = item[2], split = item[3], n_splits = item[4], part_base = item[5];
+    const int row0 = item[0], n_rows = item[1], h0 = item[2], split = item[3], n_splits = item[4], part_base = item[5], map = item[6];
     const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
-    const int M = a.maps, D = a.D, VD = a.VD, PT = a.page_tokens;
-    const int h = hm / M, map = hm - h * M;
-    const int kvh = h / (a.n_heads / a.n_kv_heads);
+    const int M = a.maps, D = a.D, VD = a.VD, PT = a.page_tokens, hpc = a.hpc;
+    const int r_c = c / hpc, h = h0 + c % hpc, hm = h * M + map;
+    const int kvh = h0 / (a.n_heads / a.n_kv_heads);
     const int key_heads = a.n_kv_heads * M, key_head = kvh * M + map;
     const int qs = (D + 31) / 32, dts = VD / 16;
     const int p0 = a.pos[row0];
     const int p_last = p0 + n_rows - 1;
     const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
-    const bool col_in = c < n_rows;
-    const int p_c = p0 + c;
+    const bool col_in = r_c < n_rows;
+    const int p_c = p0 + r_c;
     const int lo_c = lowest_seen(p_c, a.window, a.chunk);
     const int lo_min = lowest_seen(p0, a.window, a.chunk);
     const int kept_min = min(a.keep_first, lo_min);
-    const float slope = a.slopes ? a.slopes[h] : 0.0f;
+    const float slope = (a.slopes && col_in) ? a.slopes[h] : 0.0f;
+    const int hi_c = col_in ? p_c : -1;        // the highest position the column sees
+    const float inv_cap = a.softcap > 0.0f ? 1.0f / a.softcap : 0.0f;
 
     // the columns' queries: lane (c, g) holds dims 32 s + 8 g .. of column c
     bf16x8_t qf[QS];
@@ -134,7 +147,7 @@ __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
     for (int s = 0; s < QS; ++s) {
         u32x4_t v = {0u, 0u, 0u, 0u};
         if (s < qs && col_in && 32 * s + 8 * g + 8 <= D)
-            v = *(const u32x4_t*)(a.q + ((size_t)(row0 + c) * a.n_heads * M + hm) * D + 32 * s + 8 * g);
+            v = *(const u32x4_t*)(a.q + ((size_t)(row0 + r_c) * a.n_heads * M + hm) * D + 32 * s + 8 * g);
         qf[s] = __builtin_bit_cast(bf16x8_t, v);
     }
 
@@ -150,31 +163,57 @@ __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
 
     for (int ord = ord_begin; ord < ord_end; ++ord) {
         const int seg = ranges.segment(ord);
+        const int seg0 = seg * AR_SEG;
+        // the pages the segment touches (at most 9 for pages of 16 tokens): lane i holds the i-th
+        const int first_page = seg0 / PT;
+        const int my_page = (lane < 17 && first_page + lane < a.max_blocks) ? table[first_page + lane] : -1;
+        auto page_of = [&](int key) { return __shfl(my_page, key / PT - first_page); };
+        const int n_ch = min(AR_CHUNKS, (p_last - seg0) / 32 + 1);
+        auto next_chunk = [&](int ch) {     // the next chunk from ch on that some column may see keys of
+            while (ch < n_ch && seg0 + 32 * ch + 32 <= lo_min && seg0 + 32 * ch >= kept_min) ++ch;
+            return ch;
+        };
+        auto load_chunk = [&](int ch, u32x4_t (&kf)[2][QS], u32x4_t (&vf)[DT]) {
+            const int j0 = seg0 + 32 * ch;
+            const int key0 = j0 + chunk_key_r(0, c), key1 = j0 + chunk_key_r(1, c), keyv = j0 + 8 * g;
+            int page0 = page_of(key0), page1 = page_of(key1), pagev = page_of(keyv);
+            if (key0 > p_last) page0 = -1;
+            if (key1 > p_last) page1 = -1;
+            if (keyv > p_last) pagev = -1;
+            const bf16_t* k0 = a.k_cache + (((size_t)max(page0, 0) * key_heads + key_head) * PT + key0 % PT) * D + 8 * g;
+            const bf16_t* k1 = a.k_cache + (((size_t)max(page1, 0) * key_heads + key_head) * PT + key1 % PT) * D + 8 * g;
+            // values: lane (r = c, g) holds dim 16 dt + r, keys j0 + 8 g .. + 7 (one run of a transposed page)
+            const bf16_t* vbase = a.v_cache + (((size_t)max(pagev, 0) * a.n_kv_heads + kvh) * VD + c) * PT + keyv % PT;
+#pragma unroll
+            for (int s = 0; s < QS; ++s) {
+                kf[0][s] = u32x4_t{0u, 0u, 0u, 0u};
+                kf[1][s] = u32x4_t{0u, 0u, 0u, 0u};
+                if (s < qs && 32 * s + 8 * g + 8 <= D) {
+                    if (page0 >= 0) kf[0][s] = *(const u32x4_t*)(k0 + 32 * s);
+                    if (page1 >= 0) kf[1][s] = *(const u32x4_t*)(k1 + 32 * s);
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                vf[dt] = u32x4_t{0u, 0u, 0u, 0u};
+                if (dt < dts && pagev >= 0) vf[dt] = *(const u32x4_t*)(vbase + (size_t)16 * dt * PT);
+            }
+        };
         float m = -INFINITY, l = 0.0f;
         f32x4_t o[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        for (int ch = 0; ch < AR_CHUNKS; ++ch) {
-            const int j0 = seg * AR_SEG + ch * 32;
-            if (j0 > p_last) break;
-            if (j0 + 32 <= lo_min && j0 >= kept_min) continue;      // between the kept keys and the lowest seen one: no column sees any
+        // one chunk: its keys and values are in (kf, vf); the following chunk's are asked for into (kf_next, vf_next) first
+        auto work = [&](int ch, int following, const u32x4_t (&kf)[2][QS], const u32x4_t (&vf)[DT], u32x4_t (&kf_next)[2][QS], u32x4_t (&vf_next)[DT]) {
+            if (following < n_ch) load_chunk(following, kf_next, vf_next);
+            const int j0 = seg0 + 32 * ch;
             // scores of the chunk's two tiles
             f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-            {
-                const int key0 = j0 + chunk_key_r(0, c), key1 = j0 + chunk_key_r(1, c);
-                const int page0 = key0 <= p_last ? table[key0 / PT] : -1, page1 = key1 <= p_last ? table[key1 / PT] : -1;
-                const bf16_t* k0 = a.k_cache + (((size_t)max(page0, 0) * key_heads + key_head) * PT + key0 % PT) * D + 8 * g;
-                const bf16_t* k1 = a.k_cache + (((size_t)max(page1, 0) * key_heads + key_head) * PT + key1 % PT) * D + 8 * g;
 #pragma unroll
-                for (int s = 0; s < QS; ++s) {
-                    if (s < qs) {
-                        u32x4_t x0 = {0u, 0u, 0u, 0u}, x1 = {0u, 0u, 0u, 0u};
-                        const bool in = 32 * s + 8 * g + 8 <= D;
-                        if (in && page0 >= 0) x0 = *(const u32x4_t*)(k0 + 32 * s);
-                        if (in && page1 >= 0) x1 = *(const u32x4_t*)(k1 + 32 * s);
-                        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x0), qf[s], s0, 0, 0, 0);
-                        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, x1), qf[s], s1, 0, 0, 0);
-                    }
+            for (int s = 0; s < QS; ++s) {
+                if (s < qs) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[0][s]), qf[s], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[1][s]), qf[s], s1, 0, 0, 0);
                 }
             }
             // the lane's 8 scores: keys j0 + 8 g + 0 .. 7 of column c
@@ -184,9 +223,9 @@ __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
             for (int i = 0; i < 8; ++i) {
                 const int j = j0 + 8 * g + i;
                 float v = (i < 4 ? s0[i] : s1[i - 4]) * a.scale;
-                if (a.softcap > 0.0f) v = a.softcap * tanhf(v / a.softcap);
+                if (a.softcap > 0.0f) v = a.softcap * tanh_fast(v * inv_cap);
                 if (a.slopes) v = v - slope * (float)(p_c - j);
-                const bool seen = col_in && j <= p_c && (j >= lo_c || j < a.keep_first);
+                const bool seen = j <= hi_c && (j >= lo_c || j < a.keep_first);
                 x[i] = seen ? v : -INFINITY;
                 cmax = fmaxf(cmax, x[i]);
             }
@@ -210,23 +249,31 @@ __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
             bf16x8_t pf;
 #pragma unroll
             for (int i = 0; i < 8; ++i) pf[i] = (__bf16)w[i];
-            // values: lane (r = c, g) holds dim 16 dt + r, keys j0 + 8 g .. + 7 (one run of a transposed page)
-            const int keyv = j0 + 8 * g;
-            const int pagev = keyv <= p_last ? table[keyv / PT] : -1;
-            const bf16_t* vbase = a.v_cache + (((size_t)max(pagev, 0) * a.n_kv_heads + kvh) * VD + c) * PT + keyv % PT;
+            const bool rescale = __any(corr != 1.0f);     // o * 1 is o: where no column's maximum moved, the products are left out
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 if (dt < dts) {
-                    u32x4_t vv = {0u, 0u, 0u, 0u};
-                    if (pagev >= 0) vv = *(const u32x4_t*)(vbase + (size_t)16 * dt * PT);
-                    o[dt] = f32x4_t{o[dt][0] * corr, o[dt][1] * corr, o[dt][2] * corr, o[dt][3] * corr};
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pf, o[dt], 0, 0, 0);
+                    if (rescale) o[dt] = f32x4_t{o[dt][0] * corr, o[dt][1] * corr, o[dt][2] * corr, o[dt][3] * corr};
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf[dt]), pf, o[dt], 0, 0, 0);
                 }
             }
+        };
+        // two sets of operand registers take turns
+        u32x4_t kf_a[2][QS], vf_a[DT], kf_b[2][QS], vf_b[DT];
+        int ch = next_chunk(0);
+        if (ch < n_ch) load_chunk(ch, kf_a, vf_a);
+        while (ch < n_ch) {
+            int following = next_chunk(ch + 1);
+            work(ch, following, kf_a, vf_a, kf_b, vf_b);
+            ch = following;
+            if (ch >= n_ch) break;
+            following = next_chunk(ch + 1);
+            work(ch, following, kf_b, vf_b, kf_a, vf_a);
+            ch = following;
         }
-        if (part_base >= 0) {       // one column (a decoded row): its segment's sums go out as they are
-            if (c == 0) {
-                const size_t slot = (size_t)part_base + ord;
+        if (part_base >= 0) {       // a decoded row: its columns' sums of the segment go out as they are
+            if (c < hpc) {
+                const size_t slot = (size_t)part_base + (size_t)ord * hpc + c;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
                     if (dt < dts) *(f32x4_t*)(a.part_o + slot * VD + 16 * dt + 4 * g) = o[dt];
@@ -248,7 +295,7 @@ __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
         }
     }
     if (part_base >= 0 || !col_in) return;
-    const int row = row0 + c;
+    const int row = row0 + r_c;
     const Finish fin(a, row, h, Mt, Lt);
     const size_t at = ((size_t)row * a.n_heads * M + hm) * VD;
 #pragma unroll
@@ -271,28 +318,52 @@ __global__ void __launch_bounds__(64) attention_rules_kernel(RulesArgs a) {
 }
 
 // Folds the segments' sums of a decoded row's column in key order and stores its result: one wave a (row, head, map),
-// lane d owning value dims d, d + 64, ...  merges [n][4]: row, head * maps + map, first partial slot, 0.
+// lane d owning value dims d, d + 64, ...  merges [n][4]: row, head * maps + map, the column's first partial slot, slots from one
+// segment's to the next's.
 __global__ void __launch_bounds__(64) attention_rules_merge_kernel(RulesArgs a, const int* __restrict__ merges) {
     const int* mg = merges + (size_t)blockIdx.x * 4;
-    const int row = mg[0], hm = mg[1], base = mg[2];
+    const int row = mg[0], hm = mg[1], base = mg[2], stride = mg[3];
     const int lane = threadIdx.x, VD = a.VD, M = a.maps;
     const int h = hm / M;
     const int p = a.pos[row];
     const int n_ord = seg_ranges(p, p, a.window, a.keep_first, a.chunk).count();
+    // the segments' maxima and sums first (lane i asks for those of segments i, i + 64, ...), then the value sums with four
+    // segments' loads in flight; the fold itself is the tiles' chain, a segment at a time
+    __shared__ float ms[AR_MERGE_MAX], ls[AR_MERGE_MAX];
     float Mt = -INFINITY, Lt = 0.0f;
     float O[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int ord = 0; ord < n_ord; ++ord) {
-        const size_t slot = (size_t)base + ord;
-        const float m = a.part_ml[2 * slot], l = a.part_ml[2 * slot + 1];
-        float fa, fb, Mn;
-        fold_weights_r(Mt, m, fa, fb, Mn);
-        Lt = folded_r(Lt, fa, l, fb);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int d = lane + 64 * i;
-            if (d < VD) O[i] = folded_r(O[i], fa, a.part_o[slot * VD + d], fb);
+    for (int ord0 = 0; ord0 < n_ord; ord0 += AR_MERGE_MAX) {
+        const int n = min(AR_MERGE_MAX, n_ord - ord0);
+        __syncthreads();
+        for (int i = lane; i < n; i += 64) {
+            const size_t slot = (size_t)base + (size_t)(ord0 + i) * stride;
+            ms[i] = a.part_ml[2 * slot];
+            ls[i] = a.part_ml[2 * slot + 1];
         }
-        Mt = Mn;
+        __syncthreads();
+        for (int i0 = 0; i0 < n; i0 += 4) {
+            float v[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const size_t slot = (size_t)base + (size_t)(ord0 + min(i0 + u, n - 1)) * stride;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = lane + 64 * i;
+                    v[u][i] = d < VD ? a.part_o[slot * VD + d] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (i0 + u < n) {
+                    float fa, fb, Mn;
+                    fold_weights_r(Mt, ms[i0 + u], fa, fb, Mn);
+                    Lt = folded_r(Lt, fa, ls[i0 + u], fb);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) O[i] = folded_r(O[i], fa, v[u][i], fb);
+                    Mt = Mn;
+                }
+            }
+        }
     }
     const Finish fin(a, row, h, Mt, Lt);
     const size_t at = ((size_t)row * a.n_heads * M + hm) * VD;
@@ -318,14 +389,14 @@ extern "C" int llmx_attention_rules(const void* q, const void* k_cache, const vo
                                     const int* items, int n_items, const int* merges, int n_merges, void* out, int out_f32, float* part_o,
                                     float* part_ml, float scale, float softcap, int n_heads, int n_kv_heads, int maps, int head_dim, int v_dim,
                                     int page_tokens, int max_blocks, int window, int keep_first, int chunk, const float* slopes, const float* sink,
-                                    const float* gate, int gate_ld, int gate_wide, hipStream_t stream) {
+                                    const float* gate, int gate_ld, int gate_wide, int hpc, hipStream_t stream) {
     if (n_items <= 0) return 0;
     if (!llmx_attention_rules_ok(LLMX_BF16, head_dim, v_dim, page_tokens) || maps < 1 || n_heads % n_kv_heads || window < 0 || keep_first < 0 ||
-        chunk < 0 || (n_merges > 0 && (!part_o || !part_ml || !merges)) || (gate && gate_ld < (gate_wide ? n_heads * v_dim : n_heads)))
+        chunk < 0 || hpc < 1 || hpc > 16 || 16 % hpc || (hpc > 1 && hpc != n_heads / n_kv_heads) || (n_merges > 0 && (!part_o || !part_ml || !merges)) || (gate && gate_ld < (gate_wide ? n_heads * v_dim : n_heads)))
         return -2;
     RulesArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, out, out_f32, part_o, part_ml,
                 scale, softcap, n_heads, n_kv_heads, maps, head_dim, v_dim, page_tokens, max_blocks, window, keep_first, chunk, slopes, sink,
-                gate, gate_ld, gate_wide};
+                gate, gate_ld, gate_wide, hpc};
     llmx_note_launch(LK_ATTENTION_RULES);
     const int qs = (head_dim + 31) / 32, dts = v_dim / 16;
 #define LLMX_RULES(QS_, DT_) hipLaunchKernelGGL((attention_rules_kernel<QS_, DT_>), dim3(n_items), dim3(64), 0, stream, a)

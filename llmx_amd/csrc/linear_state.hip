@@ -429,11 +429,12 @@ extern "C" int llmx_head_norm_gate(const float* o, const float* w, const float* 
 //     i_t = c tanh(zi / c),  f_t = log sigmoid(c tanh(zf / c)),  m_t = max(f_t + m_(t-1), i_t)       (m starts at 0)
 //     S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,   n_t likewise with k_t alone
 // which is the scan's recurrence with one decay for all of a head's key channels, keys times exp(i_t - m_t), and one more
-// value channel that is always 1 (its column of S is n).  This kernel walks each request's rows in order for m (kept in
+// value channel that is always 1 (its column of S is n).  The preparation walks each request's rows in order for m (kept in
 // the request's state slot after the matrix, one float a head) and writes the scan's operands: decay [T, H*D], keys
 // [T, H*D], values [T, H*(V+1)], and exp(-m_t) [T, H], below which the read-out's denominator |n_t . q_t| is not let.
-// One block of 256 threads a (request, head): chunks of 256 rows; a chunk's gates are formed a thread a row, m by every
-// thread alike in row order, the exponentials a thread a row, and the rows are then written a wave a row.
+// Two launches.  The first, one block of 256 threads a (request, head), walks the request's rows in chunks of 256: a chunk's
+// gates are formed a thread a row, m by every thread alike in row order, the three exponentials a thread a row; the two
+// factors go out as [T, H, 2] (keep, take).  The second, one wave a (row, head), writes the row's operands from them.
 struct MemoryPrepArgs {
     const float* pre;        // [T, ld]: the fused projection
     int ld;
@@ -451,16 +452,17 @@ struct MemoryPrepArgs {
     float* keys;             // [T, H*D]
     float* values;           // [T, H*(V+1)]
     float* den_floor;        // [T, H]
+    float* factors;          // [T, H, 2]: keep, take
     int H, D, V;
 };
 
 #define MEM_CHUNK 256
 
-__global__ void __launch_bounds__(MEM_CHUNK) memory_prep_kernel(MemoryPrepArgs a) {
-    __shared__ float gi[MEM_CHUNK], gf[MEM_CHUNK], keep[MEM_CHUNK], take[MEM_CHUNK];
+__global__ void __launch_bounds__(MEM_CHUNK) memory_gates_kernel(MemoryPrepArgs a) {
+    __shared__ float gi[MEM_CHUNK], gf[MEM_CHUNK];
     const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int row0 = a.entry_rows[2 * e], n = a.entry_rows[2 * e + 1];
-    const int H = a.H, D = a.D, V = a.V;
+    const int H = a.H;
     float m = a.state[(size_t)a.slot_read[e] * a.state_stride + a.m_off + h];
     const float bi = a.i_bias[h], bf = a.f_bias[h];
     for (int c0 = 0; c0 < n; c0 += MEM_CHUNK) {
@@ -482,36 +484,41 @@ __global__ void __launch_bounds__(MEM_CHUNK) memory_prep_kernel(MemoryPrepArgs a
             m = now;
         }
         if (tid < rows) {
-            keep[tid] = expf(gf[tid] + mine_prev - mine_now);
-            take[tid] = expf(gi[tid] - mine_now);
-            a.den_floor[(size_t)(row0 + c0 + tid) * H + h] = expf(-mine_now);
-        }
-        __syncthreads();
-        const int wave = tid >> 6, lane = tid & 63;
-        for (int t = wave; t < rows; t += MEM_CHUNK / 64) {
-            const size_t row = (size_t)(row0 + c0 + t);
-            const float* r = a.pre + row * a.ld;
-            const float kp = keep[t], tk = take[t];
-            for (int d = lane; d < D; d += 64) {
-                a.decay[(row * H + h) * D + d] = kp;
-                a.keys[(row * H + h) * D + d] = tk * r[a.k_col + h * D + d];
-            }
-            for (int j = lane; j <= V; j += 64) a.values[(row * H + h) * (V + 1) + j] = j < V ? r[a.v_col + h * V + j] : 1.0f;
+            const size_t at = (size_t)(row0 + c0 + tid) * H + h;
+            a.factors[2 * at] = expf(gf[tid] + mine_prev - mine_now);
+            a.factors[2 * at + 1] = expf(gi[tid] - mine_now);
+            a.den_floor[at] = expf(-mine_now);
         }
         __syncthreads();
     }
     if (tid == 0) a.state[(size_t)a.slot_write[e] * a.state_stride + a.m_off + h] = m;
 }
 
+__global__ void __launch_bounds__(64) memory_rows_kernel(MemoryPrepArgs a) {
+    const size_t row = blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const int H = a.H, D = a.D, V = a.V;
+    const float* r = a.pre + row * a.ld;
+    const float kp = a.factors[2 * (row * H + h)], tk = a.factors[2 * (row * H + h) + 1];
+    for (int d = lane; d < D; d += 64) {
+        a.decay[(row * H + h) * D + d] = kp;
+        a.keys[(row * H + h) * D + d] = tk * r[a.k_col + h * D + d];
+    }
+    for (int j = lane; j <= V; j += 64) a.values[(row * H + h) * (V + 1) + j] = j < V ? r[a.v_col + h * V + j] : 1.0f;
+}
+
 extern "C" int llmx_memory_prep(const float* pre, int ld, int k_col, int v_col, int i_col, int f_col, const float* i_bias, const float* f_bias,
                                 float cap, float* state, long state_stride, int m_off, const int* slot_read, const int* slot_write,
-                                const int* entry_rows, float* decay, float* keys, float* values, float* den_floor, int n_entries, int H, int D,
-                                int V, hipStream_t stream) {
-    if (n_entries <= 0) return 0;
-    if (H < 1 || D < 1 || V < 1 || !(cap > 0.0f) || m_off < 0 || m_off + H > state_stride) return -2;
+                                const int* entry_rows, float* decay, float* keys, float* values, float* den_floor, float* factors, int rows,
+                                int n_entries, int H, int D, int V, hipStream_t stream) {
+    if (n_entries <= 0 || rows <= 0) return 0;
+    if (H < 1 || D < 1 || V < 1 || !(cap > 0.0f) || m_off < 0 || m_off + H > state_stride || !factors) return -2;
     MemoryPrepArgs a{pre, ld, k_col, v_col, i_col, f_col, i_bias, f_bias, cap, state, state_stride, m_off, slot_read, slot_write, entry_rows,
-                     decay, keys, values, den_floor, H, D, V};
+                     decay, keys, values, den_floor, factors, H, D, V};
     llmx_note_launch(LK_MEMORY_PREP);
-    hipLaunchKernelGGL(memory_prep_kernel, dim3(n_entries, H), dim3(MEM_CHUNK), 0, stream, a);
+    hipLaunchKernelGGL(memory_gates_kernel, dim3(n_entries, H), dim3(MEM_CHUNK), 0, stream, a);
+    int rc = LLMX_CHECK_LAUNCH();
+    if (rc) return rc;
+    hipLaunchKernelGGL(memory_rows_kernel, dim3(rows, H), dim3(64), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
 }

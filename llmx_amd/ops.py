@@ -91,9 +91,10 @@ def _declare(h) -> None:
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
         "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, I, P],
         "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, I, I, I, F, F, P, P],
-        "llmx_attention_rules": [P, P, P, P, P, P, P, I, P, I, P, I, P, P, F, F, I, I, I, I, I, I, I, I, I, I, P, P, P, I, I, P],
+        "llmx_attention_rules": [P, P, P, P, P, P, P, I, P, I, P, I, P, P, F, F, I, I, I, I, I, I, I, I, I, I, P, P, P, I, I, I, P],
         "llmx_attention_rules_ok": [I, I, I, I],
-        "llmx_memory_prep": [P, I, I, I, I, I, P, P, F, P, L, I, P, P, P, P, P, P, P, I, I, I, I, P],
+        "llmx_attention_rules_segment": [],
+        "llmx_memory_prep": [P, I, I, I, I, I, P, P, F, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
@@ -722,13 +723,16 @@ def head_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], gate_pre: Op
 
 def memory_prep(pre: torch.Tensor, cols: dict, i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float, state: torch.Tensor, m_off: int,
                 slot_read: torch.Tensor, slot_write: torch.Tensor, entry_rows: torch.Tensor, decay: torch.Tensor, keys: torch.Tensor,
-                values: torch.Tensor, den_floor: torch.Tensor, H: int, D: int, V: int) -> None:
+                values: torch.Tensor, den_floor: torch.Tensor, H: int, D: int, V: int, factors: Optional[torch.Tensor] = None) -> None:
     """A gated matrix memory's rows made ready for `state_scan` (see csrc/linear_state.hip): from the fused projection `pre`
     [T, ld] with k (H*D), v (H*V) and the two gates' pre-activations (H each) at the columns cols["k"], ["v"], ["i"], ["f"]:
     i = cap tanh((zi + i_bias) / cap), f = log sigmoid(cap tanh((zf + f_bias) / cap)), the running maximum m = max(f + m, i)
     of each request (kept at `m_off` of its state slot, one float a head, read at slot_read, written at slot_write);
-    decay [T, H*D] = exp(f + m_before - m), keys [T, H*D] = exp(i - m) k, values [T, H*(V+1)] = v | 1, den_floor [T, H] = exp(-m)."""
+    decay [T, H*D] = exp(f + m_before - m), keys [T, H*D] = exp(i - m) k, values [T, H*(V+1)] = v | 1, den_floor [T, H] = exp(-m).
+    `factors`: float32 [T, H, 2] of scratch (the rows' two factors on their way from the first launch to the second)."""
     T, ld = pre.shape
+    if factors is None:
+        factors = torch.empty((T, H, 2), dtype=torch.float32, device=pre.device)
     n_e = entry_rows.shape[0]
     if state.dim() != 2 or m_off + H > state.shape[1]:
         raise KernelError("memory_prep: the state does not hold the running maxima")
@@ -740,7 +744,7 @@ def memory_prep(pre: torch.Tensor, cols: dict, i_bias: torch.Tensor, f_bias: tor
                                   _dev(slot_write, "slot_write", torch.int32, (n_e,)), _dev(entry_rows, "entry_rows", torch.int32, (n_e, 2)),
                                   _dev(decay, "decay", torch.float32, (T, H * D)), _dev(keys, "keys", torch.float32, (T, H * D)),
                                   _dev(values, "values", torch.float32, (T, H * (V + 1))), _dev(den_floor, "den_floor", torch.float32, (T, H)),
-                                  n_e, H, D, V, _stream()), "memory_prep")
+                                  _dev(factors, "factors", torch.float32, (T, H, 2)), T, n_e, H, D, V, _stream()), "memory_prep")
 
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
@@ -1139,18 +1143,19 @@ class ScoreRules:
 
 class RulesPlan:
     """Work items of the matrix-core kernel that carries out ScoreRules (csrc/attention_rules.hip) for one step's rows; they
-    hold no positions.  items [n, 8] int32: first row, rows (at most 16, consecutive, of one request), head * maps + map, this
-    item's share and the number of shares its column's segments are dealt into, first slot of the segments' partial sums
-    (-1: the item folds its segments itself and stores the result); merges [n, 4]: row, head * maps + map, first slot."""
+    hold no positions.  A tile's 16 columns are `hpc` query heads for each of 16 / hpc consecutive rows of one request.
+    items [n, 8] int32: first row, rows, first head, this item's share and the number of shares its columns' segments are dealt
+    into, first slot of the segments' partial sums (-1: the item folds its segments itself and stores the result), map;
+    merges [n, 4]: row, head * maps + map, the column's first slot, slots from one segment to the next."""
 
-    def __init__(self, items, merges, n_slots, device):
+    def __init__(self, items, merges, n_slots, hpc, device):
         import numpy as np
-        self.n_items, self.n_merges, self.n_slots = len(items), len(merges), n_slots
+        self.n_items, self.n_merges, self.n_slots, self.hpc = len(items), len(merges), n_slots, hpc
         self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device) if items else None
         self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 4), device=device) if merges else None
 
 
-RULES_SEGMENT = 256          # keys in a segment of the rules kernel (its AR_SEG)
+RULES_SEGMENT = 128          # keys in a segment of the rules kernel (its AR_SEG)
 RULES_CONTEXT_STEP = 1024    # a decoded row's context is rounded up to this for its plan, so that a growing context keeps its plan (and its graph) for long
 _RULES_PLANS: dict = {}
 
@@ -1159,14 +1164,21 @@ def attention_rules_ok(dtype: torch.dtype, head_dim: int, v_dim: int, page_token
     return dtype == torch.bfloat16 and bool(lib().llmx_attention_rules_ok(BF16, int(head_dim), int(v_dim), int(page_tokens)))
 
 
-def rules_plan(row_counts, contexts, n_columns: int, device, window: int = 0, keep_first: int = 0, chunk: int = 0) -> RulesPlan:
+def rules_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, maps: int, device, window: int = 0, keep_first: int = 0,
+               chunk: int = 0) -> RulesPlan:
     """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the entry
-    holds after the step; n_columns: heads * maps.  Entries of several rows become tiles of 16 rows a (head, map); a
-    single-row entry (a decoded token) an item a (head, map), its context's segments dealt into shares when the step has few
-    rows.  How the context is shared out changes no result: segments are folded in key order either way."""
-    single = [i for i, n in enumerate(row_counts) if n == 1]
+    holds after the step.  A tile takes the query heads of one key/value head together (where their number divides 16) for
+    as many consecutive rows as 16 columns hold; a single-row entry (a decoded token) has its context's segments dealt into
+    shares when the step has few rows.  How the context is shared out changes no result: segments are folded in key order
+    either way."""
+    if lib().llmx_attention_rules_segment() != RULES_SEGMENT:
+        raise KernelError("rules_plan: the kernel library's segments are not the plan's")
+    share = n_heads // n_kv_heads
+    hpc = share if share <= 16 and 16 % share == 0 else 1
+    groups = [(h0, m) for h0 in range(0, n_heads, hpc) for m in range(maps)]
+    tile_rows = 16 // hpc
     rounded = tuple(-(-contexts[i] // RULES_CONTEXT_STEP) * RULES_CONTEXT_STEP if row_counts[i] == 1 else 0 for i in range(len(row_counts)))
-    key = (tuple(row_counts), rounded, n_columns, str(device), window, keep_first, chunk)
+    key = (tuple(row_counts), rounded, n_heads, n_kv_heads, maps, str(device), window, keep_first, chunk)
     hit = _RULES_PLANS.get(key)
     if hit is not None:
         return hit
@@ -1179,26 +1191,28 @@ def rules_plan(row_counts, contexts, n_columns: int, device, window: int = 0, ke
             whole = min(whole, chunk // RULES_SEGMENT + 2)
         return max(1, whole)
 
+    single = [i for i, n in enumerate(row_counts) if n == 1]
     n_splits = {}
     if single:
-        base = len(single) * n_columns
+        base = len(single) * len(groups)
         for i in single:
             n_splits[i] = max(1, min(segments_at_most(rounded[i]), ATTENTION_TARGET_WAVES // base))
     items, merges, slots, row = [], [], 0, 0
     for i, n in enumerate(row_counts):
         if n == 1 and n_splits[i] > 1:
             cap = segments_at_most(rounded[i])
-            for hm in range(n_columns):
+            for h0, m in groups:
                 for s in range(n_splits[i]):
-                    items.append([row, 1, hm, s, n_splits[i], slots, 0, 0])
-                merges.append([row, hm, slots, 0])
-                slots += cap
+                    items.append([row, 1, h0, s, n_splits[i], slots, m, 0])
+                for c in range(hpc):
+                    merges.append([row, (h0 + c) * maps + m, slots + c, hpc])
+                slots += cap * hpc
         else:
-            for r0 in range(0, n, 16):
-                for hm in range(n_columns):
-                    items.append([row + r0, min(16, n - r0), hm, 0, 1, -1, 0, 0])
+            for r0 in reversed(range(0, n, tile_rows)):       # the tiles with the longest contexts first: they finish last otherwise
+                for h0, m in groups:
+                    items.append([row + r0, min(tile_rows, n - r0), h0, 0, 1, -1, m, 0])
         row += n
-    plan = RulesPlan(items, merges, slots, device)
+    plan = RulesPlan(items, merges, slots, hpc, device)
     if len(_RULES_PLANS) > 256:
         _RULES_PLANS.clear()
     _RULES_PLANS[key] = plan
@@ -1269,7 +1283,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                           1 if out.dtype == torch.float32 else 0, _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale),
                                           r.softcap, n_heads, n_kv_heads, r.maps, head_dim, v_dim, page_tokens, tables.shape[1], int(window),
                                           r.keep_first, r.chunk, _dev(r.slopes, "slopes", torch.float32, (n_heads,)),
-                                          _dev(r.sink, "sink", torch.float32, (n_heads,)), gate_at, gate_ld, gate_wide, _stream()),
+                                          _dev(r.sink, "sink", torch.float32, (n_heads,)), gate_at, gate_ld, gate_wide, rules_plan.hpc, _stream()),
                "attention_rules")
         return
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,

@@ -212,7 +212,8 @@ class GatedMatrixMemory(Mixer):
         decay, keys = step.buf("memory.decay", (T, H * D), f32), step.buf("memory.keys", (T, H * D), f32)
         values, floor = step.buf("memory.values", (T, H * (V + 1)), f32), step.buf("memory.floor", (T, H), f32)
         ops.memory_prep(pre, {n: at for n, (at, _) in self.cols.items()}, self.b_i, self.b_f, self.cap, cache.state, self.state_matrix,
-                        step.entry_held_slots, step.entry_slots, step.entry_rows, decay, keys, values, floor, H, D, V)
+                        step.entry_held_slots, step.entry_slots, step.entry_rows, decay, keys, values, floor, H, D, V,
+                        factors=step.buf("memory.factors", (T, H, 2), f32))
         o = step.buf("memory.o", (T, H * (V + 1)), f32)
         ops.state_scan(view("q"), keys, values, decay, None, cache.state, step.entry_held_slots, step.entry_slots, step.entry_rows, o,
                        float(D) ** -0.5, H, H, D, V + 1, max_rows=step.max_rows_per_entry)

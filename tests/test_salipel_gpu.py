@@ -165,7 +165,7 @@ def _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, sharp=None, 
         # where the sizes allow, the matrix-core kernel for rules (its work items made for this launch's rows)
         plan = None
         if o.attention_rules_ok(dtype, D, V, page):
-            plan = o.rules_plan([n], [b], H * M, torch.device("cuda"), window, rules.keep_first, rules.chunk)
+            plan = o.rules_plan([n], [b], H, G, M, torch.device("cuda"), window, rules.keep_first, rules.chunk)
         if kind == "two_maps":
             both = torch.empty(n, H * 2 * V, device="cuda", dtype=torch.float32)
             o.paged_attention(q, kc, vc, pos, ent, tables, both, scale, H, rules=rules, rules_plan=plan)
