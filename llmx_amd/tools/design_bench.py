@@ -316,7 +316,7 @@ def measure(engine, torch, steps, warmup):
         engine.end_request(rid)
     t = min(times[1:])
     flops = prompt_flops(engine, PROMPT)
-    rec.update(prefill_tok_s=round(PROMPT / t, 1), prefill_ms=round(t * 1e3, 3), prefill_tflop=round(flops / 1e12, 2),
+    rec.update(prefill_tok_s=round(PROMPT / t, 1), prefill_ms=round(t * 1e3, 3), prefill_tflop=round(flops / 1e12, 4),
                prefill_frac=round(flops / t / BF16_PEAK, 4))
     for batch in (1, 8):
         start = CONTEXT - steps - warmup

@@ -81,17 +81,18 @@ def test_the_record_of_one_real_layer():
     assert "long" not in rec        # the long-context configuration belongs to the default run only
 
 
-def test_the_record_of_a_design_beside_its_closest_model():
-    """`--design nenotar` at a small size: one JSON line, both models with prompt and decode rates that follow from their
+@pytest.mark.parametrize("design,title", [("nenotar", "Nenotar"), ("salipel", "Salipel")])
+def test_the_record_of_a_design_beside_its_closest_model(design, title):
+    """`--design NAME` at a small size: one JSON line, both models with prompt and decode rates that follow from their
     times and fractions that follow from the work."""
-    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--design", "nenotar", "--design-sizes", "w256", "--steps", "4", "--warmup", "2"],
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--design", design, "--design-sizes", "w256", "--steps", "4", "--warmup", "2"],
                          capture_output=True, text=True, timeout=600)
     assert run.returncode == 0, run.stderr[-2000:]
     lines = [l for l in run.stdout.strip().split("\n") if l.startswith("{")]
     assert len(lines) == 1
     rec = json.loads(lines[0])
-    assert rec["design"] == "Nenotar" and rec["dtype"] == "bf16" and list(rec["sizes"]) == ["w256"]
-    for which in ("nenotar", "closest"):
+    assert rec["design"] == title and rec["dtype"] == "bf16" and list(rec["sizes"]) == ["w256"]
+    for which in (design, "closest"):
         r = rec["sizes"]["w256"][which]
         assert abs(r["prefill_tok_s"] - 2048 * 1e3 / r["prefill_ms"]) < 0.01 * r["prefill_tok_s"]
         assert abs(r["prefill_frac"] - r["prefill_tflop"] * 1e12 / (r["prefill_ms"] * 1e-3) / 2.5e15) < 2e-3
