@@ -81,7 +81,8 @@
     X(RMSNORM_ADD_NORM, "rmsnorm_add_norm")                                                                               \
     X(MEMORY_PREP, "memory_prep")                                                                                         \
     X(ATTENTION_RULES, "attention.rules")                                                                                 \
-    X(ATTENTION_RULES_MERGE, "attention.rules_merge")
+    X(ATTENTION_RULES_MERGE, "attention.rules_merge")                                                                     \
+    X(ATTENTION_RULES_SHARED, "attention.rules_shared")
 
 enum LlmxLaunchKind : int {
 #define LLMX_X(id, name) LK_##id,

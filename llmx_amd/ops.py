@@ -91,7 +91,8 @@ def _declare(h) -> None:
         "llmx_sigmoid_root": [P, P, F, P, I, I, P],
         "llmx_state_scan": [P, I, P, I, P, I, P, I, P, P, L, P, P, P, P, F, I, I, I, I, I, P, I, I, I, I, I, P],
         "llmx_head_norm_gate": [P, P, P, I, P, I, F, I, I, I, I, I, I, I, F, F, P, P],
-        "llmx_attention_rules": [P, P, P, P, P, P, P, I, P, I, P, I, P, P, F, F, I, I, I, I, I, I, I, I, I, I, P, P, P, I, I, I, P],
+        "llmx_attention_rules": [P, P, P, P, P, P, P, I, P, I, P, I, P, I, P, P, F, F, I, I, I, I, I, I, I, I, I, I, P, P, P, I, I, I, P],
+        "llmx_attention_rules_shared_ok": [I, I],
         "llmx_attention_rules_ok": [I, I, I, I],
         "llmx_attention_rules_segment": [],
         "llmx_memory_prep": [P, I, I, I, I, I, P, P, F, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
@@ -1148,9 +1149,11 @@ class RulesPlan:
     into, first slot of the segments' partial sums (-1: the item folds its segments itself and stores the result), map;
     merges [n, 4]: row, head * maps + map, the column's first slot, slots from one segment to the next."""
 
-    def __init__(self, items, merges, n_slots, hpc, device):
+    def __init__(self, items, merges, n_slots, hpc, device, group_items=()):
         import numpy as np
         self.n_items, self.n_merges, self.n_slots, self.hpc = len(items), len(merges), n_slots, hpc
+        self.n_group_items = len(group_items)       # workgroups of four tiles of consecutive rows (prompt portions)
+        self.group_items = torch.tensor(np.asarray(group_items, dtype=np.int32).reshape(-1, 8), device=device) if group_items else None
         self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device) if items else None
         self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 4), device=device) if merges else None
 
@@ -1164,13 +1167,19 @@ def attention_rules_ok(dtype: torch.dtype, head_dim: int, v_dim: int, page_token
     return dtype == torch.bfloat16 and bool(lib().llmx_attention_rules_ok(BF16, int(head_dim), int(v_dim), int(page_tokens)))
 
 
+def attention_rules_shared_ok(head_dim: int, v_dim: int) -> bool:
+    """Whether the rules kernel has its four-wave form (keys and values through LDS) for these head widths."""
+    return bool(lib().llmx_attention_rules_shared_ok(int(head_dim), int(v_dim)))
+
+
 def rules_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, maps: int, device, window: int = 0, keep_first: int = 0,
-               chunk: int = 0) -> RulesPlan:
+               chunk: int = 0, shared: bool = False) -> RulesPlan:
     """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the entry
     holds after the step.  A tile takes the query heads of one key/value head together (where their number divides 16) for
     as many consecutive rows as 16 columns hold; a single-row entry (a decoded token) has its context's segments dealt into
     shares when the step has few rows.  How the context is shared out changes no result: segments are folded in key order
-    either way."""
+    either way.  `shared`: entries of several rows go to workgroups of four tiles that bring their keys and values from
+    memory once (`attention_rules_shared_ok` says whether the kernel has that form for the head widths); the same bits."""
     if lib().llmx_attention_rules_segment() != RULES_SEGMENT:
         raise KernelError("rules_plan: the kernel library's segments are not the plan's")
     share = n_heads // n_kv_heads
@@ -1178,7 +1187,7 @@ def rules_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, maps: int, d
     groups = [(h0, m) for h0 in range(0, n_heads, hpc) for m in range(maps)]
     tile_rows = 16 // hpc
     rounded = tuple(-(-contexts[i] // RULES_CONTEXT_STEP) * RULES_CONTEXT_STEP if row_counts[i] == 1 else 0 for i in range(len(row_counts)))
-    key = (tuple(row_counts), rounded, n_heads, n_kv_heads, maps, str(device), window, keep_first, chunk)
+    key = (tuple(row_counts), rounded, n_heads, n_kv_heads, maps, str(device), window, keep_first, chunk, bool(shared))
     hit = _RULES_PLANS.get(key)
     if hit is not None:
         return hit
@@ -1197,9 +1206,13 @@ def rules_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, maps: int, d
         base = len(single) * len(groups)
         for i in single:
             n_splits[i] = max(1, min(segments_at_most(rounded[i]), ATTENTION_TARGET_WAVES // base))
-    items, merges, slots, row = [], [], 0, 0
+    items, merges, group_items, slots, row = [], [], [], 0, 0
     for i, n in enumerate(row_counts):
-        if n == 1 and n_splits[i] > 1:
+        if n > 1 and shared:
+            for r0 in reversed(range(0, n, 4 * tile_rows)):   # the longest contexts first
+                for h0, m in groups:
+                    group_items.append([row + r0, min(4 * tile_rows, n - r0), h0, 0, 1, -1, m, 0])
+        elif n == 1 and n_splits[i] > 1:
             cap = segments_at_most(rounded[i])
             for h0, m in groups:
                 for s in range(n_splits[i]):
@@ -1212,7 +1225,7 @@ def rules_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, maps: int, d
                 for h0, m in groups:
                     items.append([row + r0, min(tile_rows, n - r0), h0, 0, 1, -1, m, 0])
         row += n
-    plan = RulesPlan(items, merges, slots, hpc, device)
+    plan = RulesPlan(items, merges, slots, hpc, device, group_items)
     if len(_RULES_PLANS) > 256:
         _RULES_PLANS.clear()
     _RULES_PLANS[key] = plan
@@ -1271,7 +1284,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         gate_at, gate_ld = _rows_view(output_gate, "output_gate", rows, n_heads * v_dim)
         gate_wide = 1
     r = rules if rules is not None else ScoreRules()
-    if rules_plan is not None and rules_plan.n_items and attention_rules_ok(q.dtype, head_dim, v_dim, page_tokens):
+    if rules_plan is not None and (rules_plan.n_items or rules_plan.n_group_items) and attention_rules_ok(q.dtype, head_dim, v_dim, page_tokens):
         part_o = part_ml = None
         if rules_plan.n_slots:
             if scratch is None:
@@ -1279,6 +1292,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             part_o = scratch("attention.rules_part_o", (rules_plan.n_slots, v_dim), torch.float32)
             part_ml = scratch("attention.rules_part_ml", (rules_plan.n_slots, 2), torch.float32)
         _check(lib().llmx_attention_rules(*common, _dev(rules_plan.items, "items", torch.int32), rules_plan.n_items,
+                                          _dev(rules_plan.group_items, "group_items", torch.int32), rules_plan.n_group_items,
                                           _dev(rules_plan.merges, "merges", torch.int32), rules_plan.n_merges, _dev(out, "out"),
                                           1 if out.dtype == torch.float32 else 0, _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale),
                                           r.softcap, n_heads, n_kv_heads, r.maps, head_dim, v_dim, page_tokens, tables.shape[1], int(window),

@@ -216,9 +216,10 @@ class Attention(Mixer):
         """The work items of the matrix-core kernel for rules, made once a step and shared by every layer with the same
         columns and rules."""
         window = int(self.window or 0)
-        return step.shared(("attention.rules_plan", self.heads, self.kv_heads, self.maps, window, self.keep_first, self.chunk),
+        shared = ops.attention_rules_shared_ok(self.head_dim, self.v_dim)
+        return step.shared(("attention.rules_plan", self.heads, self.kv_heads, self.maps, window, self.keep_first, self.chunk, shared),
                            lambda: ops.rules_plan([e.n for e in step.entries], [e.past + e.n for e in step.entries], self.heads, self.kv_heads,
-                                                  self.maps, step.device, window, self.keep_first, self.chunk))
+                                                  self.maps, step.device, window, self.keep_first, self.chunk, shared=shared))
 
     def _rules_mfma(self, act, page_tokens):
         return self.special and ops.attention_rules_ok(act, self.head_dim, self.v_dim, page_tokens)

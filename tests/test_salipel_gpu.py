@@ -100,7 +100,7 @@ def _attention_weights(rng, kind, E, H, G, D, V):
     return W
 
 
-def _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, sharp=None, decode_from=None, scale=0.3, scaling=None):
+def _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, sharp=None, decode_from=None, scale=0.3, scaling=None, shared=True):
     """One attention part alone through its kernels (the step before the attention, the attention over shuffled pages, the
     join of two maps) against the plain mixer.  kind: "window" (rule = (size, keep_first)), "chunks" (rule = size) or
     "two_maps" (rule = (softcap, diff)).  sharp = (row, key): the row's query is made to fit that key alone, whether the
@@ -165,7 +165,8 @@ def _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, sharp=None, 
         # where the sizes allow, the matrix-core kernel for rules (its work items made for this launch's rows)
         plan = None
         if o.attention_rules_ok(dtype, D, V, page):
-            plan = o.rules_plan([n], [b], H, G, M, torch.device("cuda"), window, rules.keep_first, rules.chunk)
+            plan = o.rules_plan([n], [b], H, G, M, torch.device("cuda"), window, rules.keep_first, rules.chunk,
+                                shared=shared and o.attention_rules_shared_ok(D, V))
         if kind == "two_maps":
             both = torch.empty(n, H * 2 * V, device="cuda", dtype=torch.float32)
             o.paged_attention(q, kc, vc, pos, ent, tables, both, scale, H, rules=rules, rules_plan=plan)
@@ -193,8 +194,11 @@ def test_the_three_attention_forms_over_shuffled_pages(dtype, case):
     scaling = (4.0, 1.0, 4.0, 64) if R >= 16 else None
     got, want = _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, scaling=scaling)
     close(got, want, ATT_TOL[dtype], "a prompt")
-    got, want = _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, decode_from=length - 30, scaling=scaling)
-    close(got, want, ATT_TOL[dtype], "a decoded tail")
+    decoded, want = _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, decode_from=length - 30, scaling=scaling)
+    close(decoded, want, ATT_TOL[dtype], "a decoded tail")
+    # the four-wave form, the one-wave form and rows decoded alone give a row the same bits
+    alone, _ = _attention_case(dtype, kind, H, G, D, V, R, page, length, rule, scaling=scaling, shared=False)
+    assert torch.equal(alone, got) and torch.equal(decoded, got)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
@@ -482,7 +486,11 @@ def test_which_kernels_a_serving_step_takes():
         for name in ("head_norm_rope_kvwrite", "memory_prep", "state_scan", "head_norm_gate", "combine_rows", "rmsnorm",
                      "moe_combine", "route_topk"):
             assert seen.get(name), f"{dtype}: no launch of {name} ({sorted(seen)})"
-        assert seen["attention.rules" if dtype == "bfloat16" else "attention.generic"] == 2 * 4 and seen["memory_prep"] == 2 and seen["state_scan"] == 2
+        if dtype == "bfloat16":     # the prompt's portion by workgroups of four tiles, the decoded row by items and their merge
+            assert seen["attention.rules_shared"] == 4 and seen["attention.rules"] == 4
+        else:
+            assert seen["attention.generic"] == 2 * 4
+        assert seen["memory_prep"] == 2 and seen["state_scan"] == 2
         assert seen["head_norm_gate"] == 2 * 3                  # two layers of two maps and the memory's read-out
         assert seen["combine_rows"] == 2 * (4 + 1)              # every layer's join, and the side-by-side mixer's
         assert seen["rmsnorm"] >= 2 * 4                         # one norm a layer (and the model's, where a step wants rows)
